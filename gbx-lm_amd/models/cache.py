@@ -190,6 +190,7 @@ class SlotKVCache:
         self.slots.listeners.append(self)
         self.keys = None
         self.values = None
+        self.step_rows = None                     # the owner's key rows of the current step, for readers that share the table
 
     @property
     def offset(self) -> int:
@@ -248,6 +249,72 @@ class SlotKVCache:
         self.keys[slot, at] = k[idx.to(k.device)]
         if self.v_width:
             self.values[slot, at] = v[idx.to(k.device)]
+
+    def is_trimmable(self):
+        return False
+
+
+class SharedLatentRows:
+    """The cache entry of a mixer that attends over ANOTHER mixer's table (``source``, a ``SlotKVCache`` an earlier layer of the same
+    step fills): it owns no buffer and appends nothing; positions before the step come from the source's table, the step's own rows
+    from ``source.step_rows``."""
+
+    def __init__(self, source: SlotKVCache):
+        self.source = source
+        self.slots = source.slots
+
+    @property
+    def keys(self):
+        return self.source.keys
+
+    @property
+    def offset(self) -> int:
+        return self.source.offset
+
+    def ensure(self, longest: int) -> None:
+        self.source.ensure(longest)
+
+    def is_trimmable(self):
+        return False
+
+
+class SlotStateCache:
+    """What a recurrent mixer carries from token to token, for several sequences: ``state`` fp32 ``[slots, heads, dv, dk]`` (one
+    matrix per head; the key channels of one value channel lie side by side) and, for mixers with a short causal convolution in front, ``tail``
+    ``[slots, taps - 1, channels]``: the last ``taps - 1`` inputs of the convolution in the activation dtype (oldest first).  A slot
+    is not cleared when it is handed out again: a sequence whose step starts at position 0 starts from zeros (the kernels and the
+    plain path test the position, never the buffer)."""
+
+    def __init__(self, heads: int, dk: int, dv: int, channels: int = 0, taps: int = 0, slots: Optional[SequenceSlots] = None):
+        self.heads, self.dk, self.dv = int(heads), int(dk), int(dv)
+        self.channels, self.taps = int(channels), int(taps)
+        self.slots = slots if slots is not None else SequenceSlots(1)
+        self.slots.listeners.append(self)
+        self.state = None
+        self.tail = None
+
+    @property
+    def keys(self):                              # the buffer whose address a captured step depends on
+        return self.state
+
+    @property
+    def offset(self) -> int:
+        return max(self.slots.length[0], 0)
+
+    def reserve(self, dtype, device) -> None:
+        if self.state is None:
+            n = self.slots.n_slots
+            self.state = torch.zeros((n, self.heads, self.dv, self.dk), dtype=torch.float32, device=device)
+            self.tail = torch.zeros((n, max(self.taps - 1, 0), self.channels), dtype=dtype, device=device)
+
+    def grow(self, n_slots: int) -> None:
+        if self.state is not None and self.state.shape[0] < n_slots:
+            n = max(n_slots, 2 * self.state.shape[0])
+            for nm in ("state", "tail"):
+                old = getattr(self, nm)
+                new = torch.zeros((n,) + tuple(old.shape[1:]), dtype=old.dtype, device=old.device)
+                new[:old.shape[0]] = old
+                setattr(self, nm, new)
 
     def is_trimmable(self):
         return False

@@ -1,4 +1,5 @@
-"""Dense feed-forward of ragged-step models: ``down(act(up h))`` with the activation as a parameter.
+"""Dense feed-forwards of ragged-step models: ``down(act(up h))`` and the gated ``down(act(gate h) * (up h))``, activations as
+parameters.
 
 ``relu2``: the square of relu; ``gelu_tanh``: 0.5 z (1 + tanh(sqrt(2/pi) (z + 0.044715 z^3))).  The two products are plain
 matrix products (vendor library); the activation is one in-place HIP launch on GPU tensors (fp32 arithmetic, result in the
@@ -41,3 +42,37 @@ class DenseFeedForward(nn.Module):
 
     def forward(self, h: torch.Tensor) -> torch.Tensor:
         return F.linear(activate_(F.linear(h, self.up.weight), self.activation), self.down.weight)
+
+
+GLU_KINDS = ("silu", "clamped_swish")
+
+
+def glu_(gu: torch.Tensor, kind: str = "silu", limit: float = 0.0, alpha: float = 1.702) -> torch.Tensor:
+    """Rows ``gu`` [T, 2F] = gate | up  ->  [T, F] in the same dtype, fp32 arithmetic.  ``silu``: g sigmoid(g) u.  ``clamped_swish``:
+    g' = min(g, limit), u' = clamp(u, -limit, limit), g' sigmoid(alpha g') (u' + 1)."""
+    if kind not in GLU_KINDS:
+        raise ValueError(f"unknown gated activation {kind!r}")
+    if gu.is_cuda:
+        from .. import mixer_ops as M
+        return M.glu(gu, kind, limit, alpha)
+    f = gu.shape[-1] // 2
+    g, u = gu[..., :f].float(), gu[..., f:].float()
+    if kind == "silu":
+        return (F.silu(g) * u).to(gu.dtype)
+    g, u = g.clamp(max=limit), u.clamp(min=-limit, max=limit)
+    return (g * torch.sigmoid(alpha * g) * (u + 1.0)).to(gu.dtype)
+
+
+class GatedDenseFeedForward(nn.Module):
+    """``down(silu(gate h + b_g) * (up h + b_u)) + b_d``; gate and up are one product (rows gate | up)."""
+
+    def __init__(self, width: int, ff: int, bias: bool = True, kind: str = "silu"):
+        super().__init__()
+        self.ff, self.kind = ff, kind
+        self.gate_up = nn.Linear(width, 2 * ff, bias=bias)
+        self.down = nn.Linear(ff, width, bias=bias)
+        for p in self.parameters():
+            p.requires_grad_(False)
+
+    def forward(self, h: torch.Tensor) -> torch.Tensor:
+        return F.linear(glu_(F.linear(h, self.gate_up.weight, self.gate_up.bias), self.kind), self.down.weight, self.down.bias)

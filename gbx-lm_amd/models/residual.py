@@ -1,4 +1,8 @@
-"""Residual updates that normalise the BRANCH, not the stream:  x <- x + mult * rms_norm(branch) * weight.
+"""Updates of the fp32 residual stream and the norms that read it.
+
+Branch-norm form:  x <- x + mult * rms_norm(branch) * weight.  Parallel form: ``stream_add_`` / ``stream_add_norm_``.  Several
+streams (``hyper_step_``): a sublayer reads a weighted sum of ``s`` streams and its output is written to all of them while a small
+matrix mixes the streams among themselves.  ``StreamRMSNorm`` / ``StreamLayerNorm`` turn stream rows into sublayer inputs.
 
 The stream ``x`` is fp32 whatever the activation dtype is (it is a long sum of small terms); the branch arrives in the activation
 dtype, either as rows [T, W] or as ``top`` candidate rows per token [T, top, W] with fp32 mixing weights [T, top] (the routed
@@ -61,3 +65,42 @@ def stream_add_norm_(x: torch.Tensor, a: torch.Tensor, b: Optional[torch.Tensor]
         from .. import mixer_ops as M
         return M.stream_add_norm_(x, a, b, norm.weight, norm.eps)
     return norm(stream_add_(x, a, b), a.dtype)
+
+
+class StreamLayerNorm(nn.Module):
+    """Layer norm with weight and bias of fp32 stream rows into the activation dtype:  (x - mean) / sqrt(var + eps) * w + b, the
+    variance being the mean of the squared deviations."""
+
+    def __init__(self, width: int, eps: float):
+        super().__init__()
+        self.register_buffer("weight", torch.ones(width, dtype=torch.float32))
+        self.register_buffer("bias", torch.zeros(width, dtype=torch.float32))
+        self.eps = float(eps)
+
+    def forward(self, x: torch.Tensor, act_dtype: torch.dtype) -> torch.Tensor:
+        return hyper_step_(x.unsqueeze(1), None, None, None, None, None, self, act_dtype)
+
+
+def hyper_step_(streams: torch.Tensor, y: Optional[torch.Tensor], y_mix: Optional[torch.Tensor], mix: Optional[torch.Tensor],
+                write: Optional[torch.Tensor], read: Optional[torch.Tensor], norm: Optional[StreamLayerNorm],
+                act_dtype: torch.dtype) -> torch.Tensor:
+    """One sublayer boundary of a model with ``s`` residual streams, ``streams`` fp32 [T, s, W] (updated in place), as one launch:
+
+    1. if ``y`` is given (the sublayer's output, activation dtype, [T, W] -- or [T, top, W] with fp32 ``y_mix`` [T, top], whose
+       weighted sum is folded in here in fp32):  X_j <- sum_i mix[i, j] X_i + write[j] * y  for all j at once from the old streams;
+    2. u = sum_i read[i] X_i   (``read`` None: the plain sum of the streams);
+    3. returns ``norm(u)`` in ``act_dtype``, or u itself (fp32) when ``norm`` is None."""
+    if streams.is_cuda:
+        from .. import mixer_ops as M
+        return M.hyper_step_(streams, y, y_mix, mix, write, read, norm, act_dtype)
+    if y is not None:
+        z = y.float()
+        if y_mix is not None:
+            z = (z * y_mix.float().unsqueeze(-1)).sum(1)
+        streams.copy_(torch.einsum("ij,tiw->tjw", mix.float(), streams) + write.float()[None, :, None] * z[:, None, :])
+    u = streams.sum(1) if read is None else (streams * read.float()[None, :, None]).sum(1)
+    if norm is None:
+        return u
+    mean = u.mean(-1, keepdim=True)
+    var = (u - mean).pow(2).mean(-1, keepdim=True)
+    return ((u - mean) * torch.rsqrt(var + norm.eps) * norm.weight.float() + norm.bias.float()).to(act_dtype)

@@ -30,7 +30,7 @@ import torch
 import torch.nn.functional as F
 from torch import nn
 
-from .cache import SlotKVCache
+from .cache import SharedLatentRows, SlotKVCache
 from .rope_utils import rotary_table
 
 NORM_NONE, NORM_UNIT, NORM_WEIGHT = 0, 1, 2
@@ -200,17 +200,24 @@ class RotatedValueWindowAttention(nn.Module):
 
 
 class LatentAttention(nn.Module):
+    """``rot_dim = 0``: no rotated key part (attention without positions).  ``sink`` / ``gated`` False: plain softmax / no output
+    gate.  ``own_latent`` False: the mixer has no latent projection of its own and attends over the rows of ANOTHER latent mixer of
+    the same ``kv_rank`` (and rotated part) -- the table that mixer's cache holds and the rows it formed in this step, which its
+    cache hands over (``SharedLatentRows``) -- with its own queries, key and value products."""
+
     def __init__(self, width: int, heads: int, dim: int, rot_dim: int, vdim: int, kv_rank: int, rot_base: float,
-                 rot_scaling: Optional[dict], scale: float, eps: float):
+                 rot_scaling: Optional[dict], scale: float, eps: float, sink: bool = True, gated: bool = True, own_latent: bool = True):
         super().__init__()
         if rot_dim % 2:
             raise ValueError("the rotated part has an even number of channels")
         self.width, self.heads, self.dim, self.rot_dim, self.vdim, self.kv_rank = width, heads, dim, rot_dim, vdim, kv_rank
         self.scale, self.eps = float(scale), float(eps)
+        self.gated, self.own_latent = bool(gated), bool(own_latent)
         self.dk = dim + rot_dim
         self.nq, self.nl = heads * self.dk, kv_rank + rot_dim
+        self.n_own = self.nl if own_latent else 0
         # q | latent, rotated key part | gate, padded with empty rows to a multiple of 8 (rows of the product start 16-byte aligned)
-        self.inp = nn.Linear(width, (self.nq + self.nl + heads + 7) // 8 * 8, bias=False)
+        self.inp = nn.Linear(width, (self.nq + self.n_own + (heads if gated else 0) + 7) // 8 * 8, bias=False)
         # rows of every head's key product, padded with rot_dim empty rows per head (the shared rotated part is written there), then
         # the value product: one matrix product forms every head's keys and values of a whole prompt
         self.up = nn.Linear(kv_rank, heads * (self.dk + vdim), bias=False)
@@ -219,44 +226,67 @@ class LatentAttention(nn.Module):
         self.o = nn.Linear(heads * vdim, width, bias=False)
         freq, self.rot_mult = rotary_table(rot_base, rot_dim, rot_scaling)
         self.register_buffer("freq", freq)
-        self.register_buffer("latent_norm", torch.ones(kv_rank))
-        self.register_buffer("sink", torch.zeros(heads))
+        if own_latent:
+            self.register_buffer("latent_norm", torch.ones(kv_rank))
+        else:
+            self.latent_norm = None
+        if sink:
+            self.register_buffer("sink", torch.zeros(heads))
+        else:
+            self.sink = None
         for p in self.parameters():
             p.requires_grad_(False)
 
-    def make_cache(self, slots) -> SlotKVCache:
-        return SlotKVCache(self.nl, 0, None, 0, slots)
+    def make_cache(self, slots, source: Optional[SlotKVCache] = None):
+        if self.own_latent:
+            return SlotKVCache(self.nl, 0, None, 0, slots)
+        if source is None or source.k_width != self.nl or source.v_width or source.window is not None:
+            raise ValueError("a latent mixer without a latent projection needs the table of one with the same row width")
+        return SharedLatentRows(source)
 
     def fuse_weights(self, q, dkv, g, uk, uv):
-        """The module's matrices from the checkpoint's (all [out, in])."""
+        """The module's matrices from the checkpoint's (all [out, in]); ``dkv`` / ``g`` None for a mixer without them."""
         h, d, r, dv, rank = self.heads, self.dim, self.rot_dim, self.vdim, self.kv_rank
         uk_pad = torch.cat([uk.view(h, d, rank), torch.zeros((h, r, rank), dtype=uk.dtype)], dim=1).reshape(h * (d + r), rank)
-        pad = torch.zeros((self.inp.out_features - (self.nq + self.nl + h), q.shape[1]), dtype=q.dtype)
-        return {"inp.weight": torch.cat([q, dkv, g, pad]), "up.weight": torch.cat([uk_pad, uv]),
+        parts = [q] + ([dkv] if self.own_latent else []) + ([g] if self.gated else [])
+        pad = torch.zeros((self.inp.out_features - sum(p.shape[0] for p in parts), q.shape[1]), dtype=q.dtype)
+        return {"inp.weight": torch.cat(parts + [pad]), "up.weight": torch.cat([uk_pad, uv]),
                 "uk_heads": uk.view(h, d, rank).contiguous(), "uv_heads_t": uv.view(h, dv, rank).transpose(1, 2).contiguous()}
 
-    def forward(self, h: torch.Tensor, batch, cache: SlotKVCache) -> torch.Tensor:
+    def forward(self, h: torch.Tensor, batch, cache) -> torch.Tensor:
         t, hd, d, r, dv, rank = h.shape[0], self.heads, self.dim, self.rot_dim, self.vdim, self.kv_rank
         y = F.linear(h, self.inp.weight)
         pos = batch.tok[:, 1]
-        rotate_norm_heads_(y, pos, [
-            HeadSegment(0, hd, self.dk, d, r, self.freq, self.rot_mult),
-            HeadSegment(self.nq, 1, rank, norm=NORM_WEIGHT, weight=self.latent_norm),
-            HeadSegment(self.nq + rank, 1, r, 0, r, self.freq, self.rot_mult)], self.eps)
+        segments = [HeadSegment(0, hd, self.dk, d, r, self.freq, self.rot_mult)] if r else []
+        if self.own_latent:
+            segments.append(HeadSegment(self.nq, 1, rank, norm=NORM_WEIGHT, weight=self.latent_norm))
+            if r:
+                segments.append(HeadSegment(self.nq + rank, 1, r, 0, r, self.freq, self.rot_mult))
+        if segments:
+            rotate_norm_heads_(y, pos, segments, self.eps)
         q = y[:, :self.nq].view(t, hd, self.dk)
-        latent = y[:, self.nq:self.nq + self.nl]                                   # c | rotated key part: the cached row
-        gate = y[:, self.nq + self.nl:self.nq + self.nl + hd]
-        cache.reserve(max(p + n for p, n in zip(batch.pos0, batch.n_new)), y.dtype, y.device)
+        gate = y[:, self.nq + self.n_own:self.nq + self.n_own + hd] if self.gated else None
+        if self.own_latent:
+            latent = y[:, self.nq:self.nq + self.nl]                               # c | rotated key part: the cached row
+            cache.reserve(max(p + n for p, n in zip(batch.pos0, batch.n_new)), y.dtype, y.device)
+            table = cache
+        else:
+            latent, table = cache.source.step_rows, cache.source                   # the other mixer's rows of this step and its table
+            if latent is None or latent.shape[0] != t:
+                raise RuntimeError("the mixer that owns the latent rows has not run in this step")
         if not any(batch.pos0) and not batch.decode_only:           # (one-token steps always take the form below: a captured step
                                                                     # is replayed at later positions)
             kv = F.linear(latent[:, :rank], self.up.weight)
             keys = kv[:, :self.nq].view(t, hd, self.dk)
-            keys[:, :, d:] = latent[:, None, rank:]
+            if r:
+                keys[:, :, d:] = latent[:, None, rank:]
             ctx = sink_attend(q, keys, kv[:, self.nq:].view(t, hd, dv), None, batch, self.scale, None, 0, self.sink, gate)
         else:
             qa = head_project(q, self.uk_heads, r)                                 # W_uk^T q | rotated part, per head
-            mixed = sink_attend(qa, latent.view(t, 1, self.nl), latent[:, :rank].view(t, 1, rank), cache, batch, self.scale, None, 0,
+            mixed = sink_attend(qa, latent.view(t, 1, self.nl), latent[:, :rank].view(t, 1, rank), table, batch, self.scale, None, 0,
                                 self.sink, gate)
             ctx = head_project(mixed.view(t, hd, rank), self.uv_heads_t).view(t, hd * dv)
-        cache_append(cache, latent, None, batch)
+        if self.own_latent:
+            cache_append(cache, latent, None, batch)
+            cache.step_rows = latent                                # for mixers that attend over these rows later in the step
         return F.linear(ctx, self.o.weight)

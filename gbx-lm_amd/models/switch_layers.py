@@ -120,26 +120,58 @@ class SwitchGLU(nn.Module):
 class DenseRoutedGLU(nn.Module):
     """Top-k routed gated MLPs over unquantised stacked experts, rows of a ragged step in, the chosen experts' outputs out.
 
-    Router: logits in fp32 (``router`` is kept in fp32), probabilities = softmax over ALL experts, the ``top`` largest are chosen
-    (ties: the lower expert index); their mixing weights are those probabilities, divided by their sum only if ``renormalize``.
-    Expert e: down_e(silu(gate_e h) * (up_e h)); ``gate_up`` stacks gate_e over up_e as [E, 2F, K], ``down`` is [E, K, F].
+    Router, ``scoring = "softmax"``: logits in fp32 (``router`` is kept in fp32), probabilities = softmax over ALL experts, the
+    ``top`` largest are chosen (ties: the lower expert index); their mixing weights are those probabilities, divided by their sum
+    only if ``renormalize``.  ``scoring = "sigmoid"``: scores s = sigmoid(logits); the choice runs on s + ``correction`` (a vector per
+    expert that steers the choice and never the weights); with ``groups = (count, keep)`` the experts form ``count`` equal groups of
+    neighbours, a group's score is the sum of its two largest choice scores and only experts of the ``keep`` best groups can be
+    chosen; weights = the chosen s, divided by their sum (+ 1e-20) if ``renormalize``, times ``route_scale``.
+    Expert e: down_e(act(gate_e h, up_e h)); ``activation = "silu"``: silu(g) u; ``"clamped_swish"``: g' = min(g, limit), u' =
+    clamp(u, -limit, limit), g' sigmoid(1.702 g') (u' + 1).  ``gate_up`` stacks gate_e over up_e as [E, 2F, K], ``down`` is [E, K, F].
     ``forward`` returns (y [T, top, K], weights fp32 [T, top]): the weighted sum is left to the caller, which folds it into its
     normalisation / residual launch."""
 
-    def __init__(self, input_dims: int, hidden_dims: int, num_experts: int, top: int, renormalize: bool = False):
+    def __init__(self, input_dims: int, hidden_dims: int, num_experts: int, top: int, renormalize: bool = False, scoring: str = "softmax",
+                 groups=None, route_scale: float = 1.0, activation: str = "silu", limit: float = 0.0):
         super().__init__()
         if not 1 <= top <= num_experts:
             raise ValueError("top must lie in 1..num_experts")
+        if scoring not in ("softmax", "sigmoid") or activation not in ("silu", "clamped_swish"):
+            raise ValueError("unknown router scoring or expert activation")
+        if groups is not None and (num_experts % groups[0] or not 1 <= groups[1] <= groups[0] or top > groups[1] * (num_experts // groups[0])):
+            raise ValueError("groups: equal groups, 1 <= keep <= count, and the kept groups hold at least top experts")
         self.input_dims, self.hidden_dims, self.num_experts, self.top, self.renormalize = input_dims, hidden_dims, num_experts, top, renormalize
+        self.scoring, self.groups, self.route_scale = scoring, (None if groups is None else (int(groups[0]), int(groups[1]))), float(route_scale)
+        self.activation, self.limit = activation, float(limit)
         self.register_buffer("router", torch.zeros((num_experts, input_dims), dtype=torch.float32))
+        if scoring == "sigmoid":
+            self.register_buffer("correction", torch.zeros(num_experts, dtype=torch.float32))
         self.register_buffer("gate_up", torch.zeros((num_experts, 2 * hidden_dims, input_dims)))
         self.register_buffer("down", torch.zeros((num_experts, input_dims, hidden_dims)))
 
     def route(self, h: torch.Tensor):
         if h.is_cuda:
             from .. import mixer_ops as M
+            if self.scoring == "sigmoid":
+                return M.route_sigmoid_groups(h, self.router, self.correction, self.top, self.groups, self.renormalize, self.route_scale)
             return M.route_topk(h, self.router, self.top, self.renormalize)
-        probs = torch.softmax(F.linear(h.float(), self.router.float()), dim=-1)
+        logits = F.linear(h.float(), self.router.float())
+        if self.scoring == "sigmoid":
+            s = torch.sigmoid(logits)
+            c = s + self.correction.float()
+            if self.groups is not None:
+                count, keep = self.groups
+                per = c.view(c.shape[0], count, -1)
+                score = per.sort(dim=-1, descending=True).values[..., :2].sum(-1)
+                best = torch.sort(score, dim=-1, descending=True, stable=True).indices[:, :keep]
+                allowed = torch.zeros_like(score, dtype=torch.bool).scatter_(1, best, True)
+                c = torch.where(allowed[:, :, None].expand_as(per), per, torch.full_like(per, float("-inf"))).reshape(c.shape)
+            idx = torch.sort(c, dim=-1, descending=True, stable=True).indices[..., :self.top]
+            w = torch.gather(s, 1, idx)
+            if self.renormalize:
+                w = w / (w.sum(-1, keepdim=True) + 1e-20)
+            return idx.to(torch.int32), w * self.route_scale
+        probs = torch.softmax(logits, dim=-1)
         w, idx = torch.sort(probs, dim=-1, descending=True, stable=True)      # of equal experts the lower index first
         w, idx = w[..., :self.top], idx[..., :self.top]
         if self.renormalize:
@@ -150,12 +182,11 @@ class DenseRoutedGLU(nn.Module):
         idx, w = self.route(h)
         if h.is_cuda:
             from .. import mixer_ops as M
-            return M.expert_glu(h, self.gate_up, self.down, idx), w
-        f = self.hidden_dims
+            return M.expert_glu(h, self.gate_up, self.down, idx, self.activation, self.limit), w
+        from .feed_forward import glu_
         y = torch.empty((h.shape[0], self.top, self.input_dims), dtype=h.dtype, device=h.device)
         for e in range(self.num_experts):
             t, s = torch.nonzero(idx == e, as_tuple=True)
             if t.numel():
-                gu = F.linear(h[t], self.gate_up[e])
-                y[t, s] = F.linear(F.silu(gu[:, :f]) * gu[:, f:], self.down[e])
+                y[t, s] = F.linear(glu_(F.linear(h[t], self.gate_up[e]), self.activation, self.limit), self.down[e])
         return y, w

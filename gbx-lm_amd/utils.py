@@ -18,7 +18,7 @@ from typing import Any, Callable, Generator, List, Optional, Tuple, Type, Union
 import torch
 from torch import nn
 
-from .models import qdeepseek_v3, qllama, qmixtral, qphi3, qqwen2, qqwen3, qqwen3_moe, radenex, revitar
+from .models import qdeepseek_v3, qllama, qmixtral, qphi3, qqwen2, qqwen3, qqwen3_moe, radenex, revitar, tugolix
 from .models import cache as cache_mod
 from .models.quantized_linear_gba import QuantizedLinear
 from .tokenizer_utils import TokenizerWrapper, load_tokenizer
@@ -34,6 +34,7 @@ MODEL_MAPPING = {
     "qwen3_moe": qqwen3_moe,
     "radenex": radenex,       # dense checkpoint of parallel layers (latent / windowed sink attention), named by "architecture"
     "revitar": revitar,       # dense (unquantised) checkpoint; its config names itself by "architecture"
+    "tugolix": tugolix,       # dense checkpoint with several residual streams, recurrent and latent mixers, named by "architecture"
 }
 
 _DQ_KEYS = ('qstatistic', 'qscales_scales', 'qzeros_scales', 'qscales_zeros', 'qzeros_zeros')
@@ -214,7 +215,10 @@ def load_model(model_path: Path, lazy: bool = False, model_config: dict = {}, bi
             weights[k] = v.to(torch.bfloat16)
 
     model_class, model_args_class = get_model_classes(config=config)
-    model_args = model_args_class.from_dict(config)
+    args_config = config
+    if hasattr(model_class, "shapes_from"):               # sizes that only a tensor's shape gives (e.g. low ranks)
+        args_config = dict(config, shapes=model_class.shapes_from(weights, config))
+    model_args = model_args_class.from_dict(args_config)
     model = model_class(model_args)
 
     if hasattr(model, "sanitize"):
