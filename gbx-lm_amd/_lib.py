@@ -331,6 +331,17 @@ class SinkAttnArgs(ctypes.Structure):
                 ("decode_only", ctypes.c_int32), ("act", ctypes.c_int32), ("partial", ctypes.c_void_p), ("partial_splits", ctypes.c_int32)]
 
 
+class RecurrentPrepArgs(ctypes.Structure):
+    """Mirror of ``gbxm_recurrent_prep_args``."""
+    _fields_ = [("y", ctypes.c_void_p), ("y_stride", ctypes.c_int64), ("a", ctypes.c_void_p), ("a_stride", ctypes.c_int64),
+                ("conv", ctypes.c_void_p), ("tail", ctypes.c_void_p), ("decay_bias", ctypes.c_void_p), ("decay_rate", ctypes.c_void_p),
+                ("seq", ctypes.c_void_p), ("tok", ctypes.c_void_p), ("out", ctypes.c_void_p), ("out_stride", ctypes.c_int64),
+                ("T", ctypes.c_int64), ("H", ctypes.c_int32), ("G", ctypes.c_int32), ("dk", ctypes.c_int32), ("dv", ctypes.c_int32),
+                ("off_q", ctypes.c_int32), ("off_k", ctypes.c_int32), ("off_v", ctypes.c_int32), ("off_beta", ctypes.c_int32),
+                ("taps", ctypes.c_int32), ("unit", ctypes.c_int32), ("sign", ctypes.c_float), ("q_scale", ctypes.c_float),
+                ("act", ctypes.c_int32)]
+
+
 def mixers_so_path() -> str:
     return _MSO
 
@@ -376,6 +387,14 @@ def mixers() -> ctypes.CDLL:
         L.gbxm_slot_append.argtypes = [p, i64, i32, p, i64, i32, p, p, p, p, i64, i32, i32, i32, p]
         L.gbxm_sink_attention.argtypes = [ctypes.POINTER(SinkAttnArgs), p]
         L.gbxm_sink_attention_tiled.argtypes = [i32, i32, i32, i32]
+        L.gbxm_hyper_step.argtypes = [p, p, p, p, p, p, p, p, p, p, i64, i32, i32, i32, f32, i32, p]
+        L.gbxm_glu.argtypes = [p, i64, p, i64, i32, i32, f32, f32, i32, p]
+        L.gbxm_route_sigmoid_groups.argtypes = [p, p, p, p, i64, i32, i32, i32, i32, i32, f32, p]
+        L.gbxm_expert_glu_act.argtypes = [p, p, p, p, p, i64, i32, i32, i32, i32, i32, i32, f32, p, sz, p]
+        L.gbxm_recurrent_prepare.argtypes = [ctypes.POINTER(RecurrentPrepArgs), p]
+        L.gbxm_conv_tail_update.argtypes = [p, i64, p, p, i32, i32, i32, i32, p]
+        L.gbxm_state_scan.argtypes = [p, i64, p, p, p, i32, i32, i32, i32, i32, i32, p]
+        L.gbxm_head_norm_gate.argtypes = [p, p, i64, p, p, i64, i32, i32, f32, i32, i32, p]
         _mlib = L
     return _mlib
 

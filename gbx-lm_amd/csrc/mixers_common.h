@@ -47,6 +47,16 @@ template <bool FAST> __device__ __forceinline__ float sigmoid_(float x) {
 template <bool FAST> __device__ __forceinline__ float tanh_(float x) {
   if constexpr (FAST) { const float e = __expf(2.f * x); return 1.f - __fdividef(2.f, e + 1.f); } else return tanhf(x);
 }
+// Gated activations of feed-forwards (GBXM_GLU_*): silu(g) u, or the clamped form g' sigmoid(alpha g') (u' + 1) with g' = min(g, limit),
+// u' = clamp(u, -limit, limit).
+template <bool FAST> __device__ __forceinline__ float glu_act(float g, float u, int kind, float limit, float alpha) {
+  if (kind == GBXM_GLU_CLAMPED_SWISH) {
+    g = fminf(g, limit);
+    u = fminf(fmaxf(u, -limit), limit);
+    return g * sigmoid_<FAST>(alpha * g) * (u + 1.f);
+  }
+  return g * sigmoid_<FAST>(g) * u;
+}
 template <bool FAST> __device__ __forceinline__ float log1p_(float x) { if constexpr (FAST) return __logf(1.f + x); else return log1pf(x); }
 
 // floats per (split, row, head) of the key-split partial sums of softmax attention: dv sums padded to a multiple of four (rows stay

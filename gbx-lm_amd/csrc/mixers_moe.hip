@@ -41,7 +41,7 @@ __device__ __forceinline__ float lane_dot(const T* __restrict__ w, const float* 
 
 template <typename T, bool FAST, bool VEC>
 __global__ __launch_bounds__(NT) void expert_up_rows(const T* __restrict__ h, const T* __restrict__ gate_up, const int* __restrict__ idx,
-                                                    T* __restrict__ act, int K, int F, int top) {
+                                                    T* __restrict__ act, int K, int F, int top, int kind, float limit) {
   extern __shared__ float hl[];                     // the row [K]
   const int64_t pair = blockIdx.x;
   const int e = idx[pair];
@@ -55,7 +55,7 @@ __global__ __launch_bounds__(NT) void expert_up_rows(const T* __restrict__ h, co
   for (int f = blockIdx.y * FC + wave; f < f_end; f += NW) {
     const float ag = wave_sum(lane_dot<T, VEC>(wg + static_cast<int64_t>(f) * K, hl, K, lane));
     const float au = wave_sum(lane_dot<T, VEC>(wu + static_cast<int64_t>(f) * K, hl, K, lane));
-    if (lane == 0) act[pair * F + f] = from_f32<T>(ag * sigmoid_<FAST>(ag) * au);
+    if (lane == 0) act[pair * F + f] = from_f32<T>(glu_act<FAST>(ag, au, kind, limit, 1.702f));
   }
 }
 
@@ -77,8 +77,8 @@ __global__ __launch_bounds__(NT) void expert_down_rows(const T* __restrict__ act
 }
 
 template <typename T, bool FAST>
-int launch_rows(const void* h, const void* gate_up, const void* down, const int32_t* idx, void* y, int64_t P, int K, int F, int top, void* ws,
-                hipStream_t s) {
+int launch_rows(const void* h, const void* gate_up, const void* down, const int32_t* idx, void* y, int64_t P, int K, int F, int top, int kind, float limit,
+                void* ws, hipStream_t s) {
   constexpr int PER = 16 / sizeof(T);
   const bool vec = K % PER == 0 && F % PER == 0 &&
                    (reinterpret_cast<uintptr_t>(gate_up) | reinterpret_cast<uintptr_t>(down)) % 16 == 0;
@@ -88,10 +88,10 @@ int launch_rows(const void* h, const void* gate_up, const void* down, const int3
   const T* dp = static_cast<const T*>(down);
   T* act = static_cast<T*>(ws);
   if (vec) {
-    expert_up_rows<T, FAST, true><<<gu, NT, K * sizeof(float), s>>>(hp, gp, idx, act, K, F, top);
+    expert_up_rows<T, FAST, true><<<gu, NT, K * sizeof(float), s>>>(hp, gp, idx, act, K, F, top, kind, limit);
     expert_down_rows<T, true><<<gd, NT, F * sizeof(float), s>>>(act, dp, idx, static_cast<T*>(y), K, F);
   } else {
-    expert_up_rows<T, FAST, false><<<gu, NT, K * sizeof(float), s>>>(hp, gp, idx, act, K, F, top);
+    expert_up_rows<T, FAST, false><<<gu, NT, K * sizeof(float), s>>>(hp, gp, idx, act, K, F, top, kind, limit);
     expert_down_rows<T, false><<<gd, NT, F * sizeof(float), s>>>(act, dp, idx, static_cast<T*>(y), K, F);
   }
   return after_launch("expert_glu (rows)");
@@ -100,7 +100,7 @@ int launch_rows(const void* h, const void* gate_up, const void* down, const int3
 }  // namespace
 
 int launch_expert_grouped(const void* h, const void* gate_up, const void* down, const int32_t* idx, void* y, int64_t T, int K, int F, int E, int top,
-                          void* ws, size_t ws_bytes, hipStream_t s);   // mixers_moe_mfma.hip
+                          int kind, float limit, void* ws, size_t ws_bytes, hipStream_t s);   // mixers_moe_mfma.hip
 size_t expert_grouped_workspace(int64_t T, int K, int F, int E, int top);
 
 }  // namespace gbxm
@@ -117,19 +117,26 @@ extern "C" int gbxm_expert_glu_grouped(int64_t T_, int32_t K, int32_t F, int32_t
   return act == GBXM_BF16 && expert_grouped_workspace(T_, K, F, E, top) > 0;
 }
 
-extern "C" int gbxm_expert_glu(const void* h, const void* gate_up, const void* down, const int32_t* idx, void* y, int64_t T_, int32_t K, int32_t F,
-                               int32_t E, int32_t top, int32_t act, void* ws, size_t ws_bytes, void* stream) {
-  if (!h || !gate_up || !down || !idx || !y || K <= 0 || F <= 0 || E <= 0 || top < 1 || top > E || T_ < 0 || (act != GBXM_BF16 && act != GBXM_F32))
+extern "C" int gbxm_expert_glu_act(const void* h, const void* gate_up, const void* down, const int32_t* idx, void* y, int64_t T_, int32_t K,
+                                   int32_t F, int32_t E, int32_t top, int32_t act, int32_t kind, float limit, void* ws, size_t ws_bytes,
+                                   void* stream) {
+  if (!h || !gate_up || !down || !idx || !y || K <= 0 || F <= 0 || E <= 0 || top < 1 || top > E || T_ < 0 || (act != GBXM_BF16 && act != GBXM_F32) ||
+      (kind != GBXM_GLU_SILU && kind != GBXM_GLU_CLAMPED_SWISH))
     return fail(GBXM_ERR_INVALID, "expert_glu: bad argument");
   if (T_ == 0) return GBXM_OK;
   if (!ws || ws_bytes < gbxm_expert_glu_workspace(T_, K, F, E, top, act)) return fail(GBXM_ERR_INVALID, "expert_glu: workspace too small");
   hipStream_t s = static_cast<hipStream_t>(stream);
   if (act == GBXM_BF16) {
-    const int rc = launch_expert_grouped(h, gate_up, down, idx, y, T_, K, F, E, top, ws, ws_bytes, s);
+    const int rc = launch_expert_grouped(h, gate_up, down, idx, y, T_, K, F, E, top, kind, limit, ws, ws_bytes, s);
     if (rc != GBXM_ERR_UNSUPPORTED) return rc;
   }
   if (static_cast<size_t>(K > F ? K : F) * sizeof(float) > 64 * 1024) return fail(GBXM_ERR_UNSUPPORTED, "expert_glu: rows of %d channels beyond the row kernels' LDS", K > F ? K : F);
   if (T_ * top > 0x7fffffffLL || (F + FC - 1) / FC > 65535 || (K + KC - 1) / KC > 65535) return fail(GBXM_ERR_UNSUPPORTED, "expert_glu: grid");
-  return act == GBXM_BF16 ? launch_rows<bf16_t, true>(h, gate_up, down, idx, y, T_ * top, K, F, top, ws, s)
-                          : launch_rows<float, false>(h, gate_up, down, idx, y, T_ * top, K, F, top, ws, s);
+  return act == GBXM_BF16 ? launch_rows<bf16_t, true>(h, gate_up, down, idx, y, T_ * top, K, F, top, kind, limit, ws, s)
+                          : launch_rows<float, false>(h, gate_up, down, idx, y, T_ * top, K, F, top, kind, limit, ws, s);
+}
+
+extern "C" int gbxm_expert_glu(const void* h, const void* gate_up, const void* down, const int32_t* idx, void* y, int64_t T_, int32_t K, int32_t F,
+                               int32_t E, int32_t top, int32_t act, void* ws, size_t ws_bytes, void* stream) {
+  return gbxm_expert_glu_act(h, gate_up, down, idx, y, T_, K, F, E, top, act, GBXM_GLU_SILU, 0.f, ws, ws_bytes, stream);
 }

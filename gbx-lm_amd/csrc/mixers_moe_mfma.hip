@@ -76,7 +76,7 @@ struct BTile {
 
 __global__ __launch_bounds__(256) void expert_up_kernel(const bf16_t* __restrict__ h, const bf16_t* __restrict__ gate_up, const int* __restrict__ offsets,
                                                        const int* __restrict__ sorted, const int* __restrict__ tile_tab, bf16_t* __restrict__ act,
-                                                       int K, int F, int top) {
+                                                       int K, int F, int top, int kind, float limit) {
   __shared__ __attribute__((aligned(16))) unsigned char bl[RT * BROW];
   const int bt = xcd_row_tile();
   const int e = tile_tab[2 * bt];
@@ -140,7 +140,7 @@ __global__ __launch_bounds__(256) void expert_up_kernel(const bf16_t* __restrict
     for (int q4 = 0; q4 < 4; ++q4) {
       float v[4];
 #pragma unroll
-      for (int i = 0; i < 4; ++i) { const float g = ag[j][4 * q4 + i]; v[i] = g * sigmoid_<true>(g) * au[j][4 * q4 + i]; }
+      for (int i = 0; i < 4; ++i) { const float g = ag[j][4 * q4 + i]; v[i] = glu_act<true>(g, au[j][4 * q4 + i], kind, limit, 1.702f); }
       *reinterpret_cast<u32x2*>(ap + 8 * q4) = u32x2{pack2(v[0], v[1]), pack2(v[2], v[3])};
     }
   }
@@ -236,7 +236,7 @@ size_t expert_grouped_workspace(int64_t T, int K, int F, int E, int top) {
 }
 
 int launch_expert_grouped(const void* h, const void* gate_up, const void* down, const int32_t* idx, void* y, int64_t T, int K, int F, int E, int top,
-                          void* ws, size_t ws_bytes, hipStream_t s) {
+                          int kind, float limit, void* ws, size_t ws_bytes, hipStream_t s) {
   const size_t need = expert_grouped_workspace(T, K, F, E, top);
   if (need == 0) return GBXM_ERR_UNSUPPORTED;
   if (ws_bytes < need) return fail(GBXM_ERR_INVALID, "expert_glu: workspace of %zu bytes, %zu needed", ws_bytes, need);
@@ -255,7 +255,7 @@ int launch_expert_grouped(const void* h, const void* gate_up, const void* down, 
   bf16_t* act = reinterpret_cast<bf16_t*>(w);
   expert_sort_kernel<<<1, 1024, (3 * E + 1) * sizeof(int), s>>>(idx, offsets, sorted, tile_tab, tiles, P, E);
   expert_up_kernel<<<dim3(tiles, (F + 127) / 128), 256, 0, s>>>(static_cast<const bf16_t*>(h), static_cast<const bf16_t*>(gate_up), offsets, sorted,
-                                                                 tile_tab, act, K, F, top);
+                                                                 tile_tab, act, K, F, top, kind, limit);
   expert_down_kernel<<<dim3(tiles, (K + 255) / 256), 256, 0, s>>>(act, static_cast<const bf16_t*>(down), offsets, sorted, tile_tab,
                                                                    static_cast<bf16_t*>(y), K, F);
   return after_launch("expert_glu (grouped)");

@@ -1,0 +1,268 @@
+// Recurrent mixers: a decayed matrix state per head.
+//
+//   recurrent_prep_kernel   one workgroup per row: short causal convolution + silu on q | k | v, unit q / k heads, q scale, the decay
+//                           exp(-rate_h softplus(sign (a + bias))) and beta = sigmoid(b), all in fp32, into one fp32 row.
+//   conv_tail_kernel        the last taps-1 convolution inputs of every sequence into its slot.
+//   state_scan_kernel<R>    the scan.  The columns of a head's state (one per value channel) never meet: a wave takes four columns, 16
+//                           lanes per column, a lane holds R neighbouring key channels of its column in registers; per token the two
+//                           dot products over key channels are R multiply-adds and four cross-lane adds inside a 16-lane row (all 16
+//                           lanes end with the same bits).  The next token's operands are fetched while the current one is computed.
+//                           Sums run in a fixed order: a sequence's result does not depend on what else is in the step.
+//   head_norm_gate_kernel   per-head RMS norm of the read-out, weight and gate, one wave per (row, head).
+#include "mixers_common.h"
+
+namespace gbxm {
+namespace {
+
+constexpr int NT = 256, NW = NT / 64;
+
+template <typename T, bool FAST>
+__global__ __launch_bounds__(NT) void recurrent_prep_kernel(gbxm_recurrent_prep_args p) {
+  extern __shared__ float row[];            // q | k | v of the row after convolution and silu
+  const int64_t t = blockIdx.x;
+  const int b = p.tok[2 * t], pos = p.tok[2 * t + 1];
+  const int slot = p.seq[4 * b], pos0 = p.seq[4 * b + 1], row0 = p.seq[4 * b + 3];
+  const int nq = p.G * p.dk, nv = p.H * p.dv, nd = p.H * p.dk;
+  const int C = 2 * nq + nv;
+  const T* y = static_cast<const T*>(p.y);
+  const T* yr = y + t * p.y_stride;
+  float* out = p.out + t * p.out_stride;
+  if (p.conv) {
+    const T* cw = static_cast<const T*>(p.conv);
+    const T* tail = static_cast<const T*>(p.tail) + static_cast<int64_t>(slot) * (p.taps - 1) * C;
+    for (int c = threadIdx.x; c < C; c += NT) {
+      float acc = 0.f;
+      for (int j = 0; j < p.taps; ++j) {
+        const int src = pos - (p.taps - 1) + j;
+        if (src < 0) continue;
+        const float x = src >= pos0 ? to_f32(y[(row0 + (src - pos0)) * p.y_stride + p.off_q + c])
+                                    : to_f32(tail[static_cast<int64_t>(src - pos0 + p.taps - 1) * C + c]);
+        acc += to_f32(cw[c * p.taps + j]) * x;
+      }
+      row[c] = acc * sigmoid_<FAST>(acc);
+    }
+  } else {
+    for (int c = threadIdx.x; c < nq; c += NT) { row[c] = to_f32(yr[p.off_q + c]); row[nq + c] = to_f32(yr[p.off_k + c]); }
+    for (int c = threadIdx.x; c < nv; c += NT) row[2 * nq + c] = to_f32(yr[p.off_v + c]);
+  }
+  __syncthreads();
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  // q and k heads: a wave per head
+  for (int hd = wave; hd < 2 * p.G; hd += NW) {
+    const float* v = row + hd * p.dk;
+    float mul = hd < p.G ? p.q_scale : 1.f;
+    if (p.unit) {
+      float ss = 0.f;
+      for (int c = lane; c < p.dk; c += 64) ss += v[c] * v[c];
+      mul *= 1.f / sqrtf(wave_sum(ss) + 1e-6f);
+    }
+    for (int c = lane; c < p.dk; c += 64) out[hd * p.dk + c] = v[c] * mul;
+  }
+  for (int c = threadIdx.x; c < nv; c += NT) out[2 * nq + c] = row[2 * nq + c];
+  const T* ar = static_cast<const T*>(p.a) + t * p.a_stride;
+  for (int c = threadIdx.x; c < nd; c += NT) {
+    const float z = p.sign * (to_f32(ar[c]) + p.decay_bias[c]);
+    const float sp = z > 20.f ? z : log1p_<FAST>(exp_<FAST>(z));
+    out[2 * nq + nv + c] = exp_<FAST>(-p.decay_rate[c / p.dk] * sp);
+  }
+  if (p.off_beta >= 0)
+    for (int c = threadIdx.x; c < p.H; c += NT) out[2 * nq + nv + nd + c] = sigmoid_<FAST>(to_f32(yr[p.off_beta + c]));
+}
+
+template <typename T>
+__global__ __launch_bounds__(NT) void conv_tail_kernel(const T* __restrict__ y, int64_t y_stride, T* __restrict__ tail, const int* __restrict__ seq,
+                                                      int C, int taps) {
+  const int b = blockIdx.y;
+  const int slot = seq[4 * b], pos0 = seq[4 * b + 1], n = seq[4 * b + 2], row0 = seq[4 * b + 3];
+  const int keep = taps - 1;
+  T* tl = tail + static_cast<int64_t>(slot) * keep * C;
+  for (int c = blockIdx.x * NT + threadIdx.x; c < C; c += gridDim.x * NT) {
+    // entry i afterwards holds position pos0 + n - keep + i: ascending i reads entries above the ones already written
+    for (int i = 0; i < keep; ++i) {
+      const int pos = pos0 + n - keep + i;
+      T v;
+      if (pos >= pos0) v = y[(row0 + (pos - pos0)) * y_stride + c];
+      else if (pos >= 0) v = tl[static_cast<int64_t>(i + n) * C + c];
+      else v = from_f32<T>(0.f);
+      tl[static_cast<int64_t>(i) * C + c] = v;
+    }
+  }
+}
+
+// Sum over the 16 lanes of a row; every lane of the row gets the same bits (each step adds the two halves of a mirrored pair).
+__device__ __forceinline__ float row16_sum(float v) {
+  v += __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), 0xB1, 0xf, 0xf, false));    // quad_perm [1,0,3,2]
+  v += __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), 0x4E, 0xf, 0xf, false));    // quad_perm [2,3,0,1]
+  v += __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), 0x141, 0xf, 0xf, false));   // row_half_mirror
+  v += __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), 0x140, 0xf, 0xf, false));   // row_mirror
+  return v;
+}
+
+template <int R, bool DELTA>
+__global__ __launch_bounds__(64) void state_scan_kernel(const float* __restrict__ r, int64_t r_stride, float* __restrict__ state,
+                                                       float* __restrict__ out, const int* __restrict__ seq, int H, int G, int dk, int dv) {
+  const int b = blockIdx.z, h = blockIdx.y;
+  const int lane = threadIdx.x, ks = lane & 15;
+  const int col = blockIdx.x * 4 + (lane >> 4);
+  const int slot = seq[4 * b], pos0 = seq[4 * b + 1], n = seq[4 * b + 2], row0 = seq[4 * b + 3];
+  const bool col_ok = col < dv;
+  const int colc = col_ok ? col : dv - 1;
+  const int c0 = ks * R;
+  const int nq = G * dk, nv = H * dv;
+  const int g = h / (H / G);
+  float* sp = state + ((static_cast<int64_t>(slot) * H + h) * dv + colc) * dk + c0;
+  float S[R];
+#pragma unroll
+  for (int i = 0; i < R; ++i) S[i] = (pos0 > 0 && c0 + i < dk) ? sp[i] : 0.f;
+  const float* base = r + static_cast<int64_t>(row0) * r_stride;
+  const int oq = g * dk + c0, ok = nq + g * dk + c0, ov = 2 * nq + h * dv + colc, og = 2 * nq + nv + h * dk + c0, ob = 2 * nq + nv + H * dk + h;
+  float q[R], k[R], d[R], v, beta = 1.f;
+  auto fetch = [&](const float* rp, float* fq, float* fk, float* fd, float& fv, float& fb) {
+#pragma unroll
+    for (int i = 0; i < R; ++i) {
+      const bool in = c0 + i < dk;
+      fq[i] = in ? rp[oq + i] : 0.f;
+      fk[i] = in ? rp[ok + i] : 0.f;
+      fd[i] = in ? rp[og + i] : 1.f;
+    }
+    fv = rp[ov];
+    if constexpr (DELTA) fb = rp[ob];
+  };
+  fetch(base, q, k, d, v, beta);
+  float* op = out + static_cast<int64_t>(row0) * nv + h * dv + colc;
+  for (int t = 0; t < n; ++t) {
+    float nq_[R], nk_[R], nd_[R], nv_ = 0.f, nb_ = 1.f;
+    const bool more = t + 1 < n;
+    if (more) fetch(base + static_cast<int64_t>(t + 1) * r_stride, nq_, nk_, nd_, nv_, nb_);
+    float u = v;
+#pragma unroll
+    for (int i = 0; i < R; ++i) S[i] *= d[i];
+    if constexpr (DELTA) {
+      float dot = 0.f;
+#pragma unroll
+      for (int i = 0; i < R; ++i) dot += k[i] * S[i];
+      u = beta * (v - row16_sum(dot));
+    }
+    float o = 0.f;
+#pragma unroll
+    for (int i = 0; i < R; ++i) { S[i] += k[i] * u; o += q[i] * S[i]; }
+    o = row16_sum(o);
+    if (ks == 0 && col_ok) op[static_cast<int64_t>(t) * nv] = o;
+    if (more) {
+#pragma unroll
+      for (int i = 0; i < R; ++i) { q[i] = nq_[i]; k[i] = nk_[i]; d[i] = nd_[i]; }
+      v = nv_;
+      beta = nb_;
+    }
+  }
+  if (col_ok) {
+#pragma unroll
+    for (int i = 0; i < R; ++i)
+      if (c0 + i < dk) sp[i] = S[i];
+  }
+}
+
+template <typename T, bool FAST>
+__global__ __launch_bounds__(NT) void head_norm_gate_kernel(const float* __restrict__ o, const T* __restrict__ gate, int64_t gate_stride,
+                                                           const float* __restrict__ w, T* __restrict__ out, int H, int dv, float eps, int kind) {
+  const int64_t t = blockIdx.x;
+  const int lane = threadIdx.x & 63;
+  const int h = blockIdx.y * NW + (threadIdx.x >> 6);
+  if (h >= H) return;
+  const float* x = o + (t * H + h) * dv;
+  float ss = 0.f;
+  for (int c = lane; c < dv; c += 64) ss += x[c] * x[c];
+  const float r = 1.f / sqrtf(wave_sum(ss) / dv + eps);
+  const T* g = gate + t * gate_stride + h * dv;
+  T* y = out + (t * H + h) * dv;
+  for (int c = lane; c < dv; c += 64) {
+    const float z = to_f32(g[c]);
+    const float s = sigmoid_<FAST>(z);
+    y[c] = from_f32<T>(x[c] * r * w[c] * (kind == 1 ? z * s : s));
+  }
+}
+
+template <bool DELTA>
+int launch_scan(int R, dim3 grid, hipStream_t s, const float* r, int64_t r_stride, float* state, float* out, const int32_t* seq, int H, int G, int dk,
+                int dv) {
+#define GBXM_SCAN(N) state_scan_kernel<N, DELTA><<<grid, 64, 0, s>>>(r, r_stride, state, out, seq, H, G, dk, dv)
+  if (R <= 1) GBXM_SCAN(1);
+  else if (R <= 2) GBXM_SCAN(2);
+  else if (R <= 3) GBXM_SCAN(3);
+  else if (R <= 4) GBXM_SCAN(4);
+  else if (R <= 6) GBXM_SCAN(6);
+  else if (R <= 8) GBXM_SCAN(8);
+  else if (R <= 12) GBXM_SCAN(12);
+  else GBXM_SCAN(16);
+#undef GBXM_SCAN
+  return after_launch("state_scan");
+}
+
+bool act_ok(int act) { return act == GBXM_BF16 || act == GBXM_F32; }
+
+}  // namespace
+}  // namespace gbxm
+
+using namespace gbxm;
+
+extern "C" {
+
+int gbxm_recurrent_prepare(const gbxm_recurrent_prep_args* a, void* stream) {
+  if (!a || !act_ok(a->act) || !a->y || !a->a || !a->decay_bias || !a->decay_rate || !a->seq || !a->tok || !a->out || a->T < 0 || a->H < 1 || a->G < 1 ||
+      a->H % a->G || a->dk < 1 || a->dv < 1 || a->off_q < 0 || a->off_k < 0 || a->off_v < 0)
+    return fail(GBXM_ERR_INVALID, "recurrent_prepare: bad argument");
+  const int nq = a->G * a->dk, nv = a->H * a->dv, C = 2 * nq + nv;
+  if (a->conv && (a->taps < 1 || (a->taps > 1 && !a->tail) || a->off_k != a->off_q + nq || a->off_v != a->off_k + nq))
+    return fail(GBXM_ERR_INVALID, "recurrent_prepare: a convolution needs q | k | v side by side and the slots' tails");
+  if (a->out_stride < C + a->H * a->dk + (a->off_beta >= 0 ? a->H : 0)) return fail(GBXM_ERR_INVALID, "recurrent_prepare: output rows too short");
+  const size_t lds = static_cast<size_t>(C) * sizeof(float);
+  if (lds > 60 * 1024) return fail(GBXM_ERR_UNSUPPORTED, "recurrent_prepare: q | k | v rows of %d channels", C);
+  if (a->T == 0) return GBXM_OK;
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  if (a->act == GBXM_BF16) recurrent_prep_kernel<bf16_t, false><<<dim3(a->T), NT, lds, s>>>(*a);
+  else recurrent_prep_kernel<float, false><<<dim3(a->T), NT, lds, s>>>(*a);
+  return after_launch("recurrent_prepare");
+}
+
+int gbxm_conv_tail_update(const void* y, int64_t y_stride, void* tail, const int32_t* seq, int32_t B, int32_t C, int32_t taps, int32_t act,
+                          void* stream) {
+  if (!act_ok(act) || !y || !tail || !seq || B < 0 || C < 1 || taps < 2 || y_stride < C) return fail(GBXM_ERR_INVALID, "conv_tail_update: bad argument");
+  if (B == 0) return GBXM_OK;
+  if (B > 65535) return fail(GBXM_ERR_UNSUPPORTED, "conv_tail_update: more than 65535 sequences in a step");
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  const dim3 grid((C + NT - 1) / NT, B);
+  if (act == GBXM_BF16) conv_tail_kernel<bf16_t><<<grid, NT, 0, s>>>(static_cast<const bf16_t*>(y), y_stride, static_cast<bf16_t*>(tail), seq, C, taps);
+  else conv_tail_kernel<float><<<grid, NT, 0, s>>>(static_cast<const float*>(y), y_stride, static_cast<float*>(tail), seq, C, taps);
+  return after_launch("conv_tail_update");
+}
+
+int gbxm_state_scan(const float* r, int64_t r_stride, float* state, float* out, const int32_t* seq, int32_t B, int32_t H, int32_t G, int32_t dk,
+                    int32_t dv, int32_t delta, void* stream) {
+  if (!r || !state || !out || !seq || B < 0 || H < 1 || G < 1 || H % G || dk < 1 || dv < 1 ||
+      r_stride < 2 * G * dk + H * dv + H * dk + (delta ? H : 0))
+    return fail(GBXM_ERR_INVALID, "state_scan: bad argument");
+  if (dk > 256) return fail(GBXM_ERR_UNSUPPORTED, "state_scan: %d key channels per head (at most 256)", dk);
+  if (B == 0) return GBXM_OK;
+  if (B > 65535 || H > 65535) return fail(GBXM_ERR_UNSUPPORTED, "state_scan: grid");
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  const dim3 grid((dv + 3) / 4, H, B);
+  const int R = (dk + 15) / 16;
+  return delta ? launch_scan<true>(R, grid, s, r, r_stride, state, out, seq, H, G, dk, dv)
+               : launch_scan<false>(R, grid, s, r, r_stride, state, out, seq, H, G, dk, dv);
+}
+
+int gbxm_head_norm_gate(const float* o, const void* gate, int64_t gate_stride, const float* w, void* out, int64_t T_, int32_t H, int32_t dv,
+                        float eps, int32_t kind, int32_t act, void* stream) {
+  if (!act_ok(act) || !o || !gate || !w || !out || T_ < 0 || H < 1 || dv < 1 || gate_stride < H * dv || (kind != 1 && kind != 2))
+    return fail(GBXM_ERR_INVALID, "head_norm_gate: bad argument");
+  if (T_ == 0) return GBXM_OK;
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  const dim3 grid(T_, (H + NW - 1) / NW);
+  if (act == GBXM_BF16)
+    head_norm_gate_kernel<bf16_t, false><<<grid, NT, 0, s>>>(o, static_cast<const bf16_t*>(gate), gate_stride, w, static_cast<bf16_t*>(out), H, dv, eps, kind);
+  else
+    head_norm_gate_kernel<float, false><<<grid, NT, 0, s>>>(o, static_cast<const float*>(gate), gate_stride, w, static_cast<float*>(out), H, dv, eps, kind);
+  return after_launch("head_norm_gate");
+}
+
+}  // extern "C"

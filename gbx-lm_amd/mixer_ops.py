@@ -98,7 +98,11 @@ def route_topk(h: torch.Tensor, router: torch.Tensor, top: int, renormalize: boo
     return idx, w
 
 
-def expert_glu(h: torch.Tensor, gate_up: torch.Tensor, down: torch.Tensor, idx: torch.Tensor) -> torch.Tensor:
+_GLU = {"silu": 1, "clamped_swish": 2}
+
+
+def expert_glu(h: torch.Tensor, gate_up: torch.Tensor, down: torch.Tensor, idx: torch.Tensor, activation: str = "silu",
+               limit: float = 0.0) -> torch.Tensor:
     act = _act(h, "h")
     h = h.contiguous()
     t, k = h.shape
@@ -112,8 +116,8 @@ def expert_glu(h: torch.Tensor, gate_up: torch.Tensor, down: torch.Tensor, idx: 
     L = _lib.mixers()
     nbytes = L.gbxm_expert_glu_workspace(t, k, f, e, top, act)
     ws = torch.empty((nbytes,), dtype=torch.uint8, device=h.device) if nbytes else None
-    _lib.check_mixers(L.gbxm_expert_glu(h.data_ptr(), gate_up.data_ptr(), down.data_ptr(), idx.data_ptr(), y.data_ptr(), t, k, f, e, top, act,
-                                        None if ws is None else ws.data_ptr(), nbytes, _stream(h.device)))
+    _lib.check_mixers(L.gbxm_expert_glu_act(h.data_ptr(), gate_up.data_ptr(), down.data_ptr(), idx.data_ptr(), y.data_ptr(), t, k, f, e, top, act,
+                                            _GLU[activation], float(limit), None if ws is None else ws.data_ptr(), nbytes, _stream(h.device)))
     return y
 
 
@@ -290,4 +294,131 @@ def sink_attention(q: torch.Tensor, k_new: torch.Tensor, v_new: torch.Tensor, ca
             partial = torch.empty((splits, t, heads, (dv + 3) // 4 * 4 + 4), dtype=torch.float32, device=q.device)
             a.partial, a.partial_splits = partial.data_ptr(), splits
     _lib.check_mixers(_lib.mixers().gbxm_sink_attention(ctypes.byref(a), _stream(q.device)))
+    return out
+
+
+# ------------------------------------------------------------------------------- several streams, gated activations, grouped sigmoid router
+def hyper_step_(streams: torch.Tensor, y: Optional[torch.Tensor], y_mix: Optional[torch.Tensor], mix: Optional[torch.Tensor],
+                write: Optional[torch.Tensor], read: Optional[torch.Tensor], norm, act_dtype: torch.dtype) -> torch.Tensor:
+    """models/residual.py:hyper_step_ as one launch.  streams fp32 [T, S, W] contiguous, updated in place."""
+    if not streams.is_cuda or streams.dim() != 3:
+        raise RuntimeError("gbx_lm_amd.mixer_ops: hyper_step_ takes fp32 device streams [T, S, W]")
+    _f32(streams, "streams")
+    t, s, width = streams.shape
+    top = 1
+    if y is not None:
+        if y.dtype != act_dtype or not y.is_contiguous():
+            raise TypeError("hyper_step_: the sublayer's output must be contiguous and in the activation dtype")
+        top = 1 if y_mix is None else y_mix.shape[-1]
+        if y.numel() != t * top * width or mix.shape != (s, s) or write.numel() != s:
+            raise ValueError("hyper_step_: shapes do not fit")
+    if read is not None and read.numel() != s:
+        raise ValueError("hyper_step_: one read weight per stream")
+    ptr = lambda x, nm: None if x is None else _f32(x, nm).data_ptr()
+    h = u = None
+    if norm is not None:
+        if norm.weight.numel() != width or norm.bias.numel() != width:
+            raise ValueError("hyper_step_: one norm weight and bias per channel")
+        h = torch.empty((t, width), dtype=act_dtype, device=streams.device)
+    else:
+        u = torch.empty((t, width), dtype=torch.float32, device=streams.device)
+    _lib.check_mixers(_lib.mixers().gbxm_hyper_step(
+        streams.data_ptr(), None if y is None else y.data_ptr(), ptr(y_mix, "y_mix"), ptr(mix, "mix"), ptr(write, "write"), ptr(read, "read"),
+        None if norm is None else _f32(norm.weight, "norm.weight").data_ptr(), None if norm is None else _f32(norm.bias, "norm.bias").data_ptr(),
+        None if h is None else h.data_ptr(), None if u is None else u.data_ptr(), t, s, width, top, 0.0 if norm is None else float(norm.eps),
+        _DT[act_dtype], _stream(streams.device)))
+    return h if norm is not None else u
+
+
+def glu(gu: torch.Tensor, kind: str, limit: float = 0.0, alpha: float = 1.702) -> torch.Tensor:
+    act = _act(gu, "gu")
+    if gu.dim() != 2 or gu.stride(1) != 1 or gu.shape[1] % 2:
+        raise ValueError("glu: rows [T, 2F] with unit inner stride")
+    t, f = gu.shape[0], gu.shape[1] // 2
+    out = torch.empty((t, f), dtype=gu.dtype, device=gu.device)
+    _lib.check_mixers(_lib.mixers().gbxm_glu(gu.data_ptr(), gu.stride(0), out.data_ptr(), t, f, _GLU[kind], float(limit), float(alpha), act,
+                                            _stream(gu.device)))
+    return out
+
+
+def route_sigmoid_groups(h: torch.Tensor, router: torch.Tensor, correction: torch.Tensor, top: int, groups, renormalize: bool, scale: float):
+    """(idx int32 [T, top], weights fp32 [T, top]).  The logits are an fp32 product of the rows (their bf16 image widened, when
+    activations are bf16) with the fp32 router (vendor library); scores, groups and the choice are one launch."""
+    _act(h, "h")
+    logits = torch.matmul(h if h.dtype == torch.float32 else h.float(), _f32(router, "router").t())
+    t, e = logits.shape
+    idx = torch.empty((t, top), dtype=torch.int32, device=h.device)
+    w = torch.empty((t, top), dtype=torch.float32, device=h.device)
+    count, keep = groups if groups is not None else (0, 0)
+    _lib.check_mixers(_lib.mixers().gbxm_route_sigmoid_groups(logits.data_ptr(), _f32(correction, "correction").data_ptr(), idx.data_ptr(), w.data_ptr(),
+                                                             t, e, top, count, keep, int(bool(renormalize)), float(scale), _stream(h.device)))
+    return idx, w
+
+
+# ------------------------------------------------------------------------------- recurrent mixers (models/recurrent_mixers.py)
+def recurrent_prepare(y: torch.Tensor, a: torch.Tensor, lay, decay_bias: torch.Tensor, decay_rate: torch.Tensor, sign: float,
+                      conv: Optional[torch.Tensor], cache, batch, unit: bool, q_scale: float) -> torch.Tensor:
+    act = _act(y, "y")
+    t = y.shape[0]
+    if y.dim() != 2 or y.stride(1) != 1 or a.dim() != 2 or a.stride(1) != 1 or a.dtype != y.dtype or a.shape != (t, lay.nd) or t != batch.total:
+        raise ValueError("recurrent_prepare: projection rows do not fit the step")
+    if max(lay.off_q + lay.nq, lay.off_k + lay.nq, lay.off_v + lay.nv, lay.off_beta + lay.heads) > y.shape[1]:
+        raise ValueError("recurrent_prepare: the layout ends outside the rows")
+    if decay_bias.numel() != lay.nd or decay_rate.numel() != lay.heads:
+        raise ValueError("recurrent_prepare: one decay bias per head and key channel, one rate per head")
+    out = torch.empty((t, lay.out_width), dtype=torch.float32, device=y.device)
+    p = _lib.RecurrentPrepArgs()
+    p.y, p.y_stride, p.a, p.a_stride = y.data_ptr(), y.stride(0), a.data_ptr(), a.stride(0)
+    p.conv = p.tail = None
+    p.taps = 0
+    if conv is not None:
+        c = 2 * lay.nq + lay.nv
+        if conv.dtype != y.dtype or not conv.is_contiguous() or conv.shape[0] != c:
+            raise ValueError("recurrent_prepare: convolution taps [q | k | v channels, taps] in the activation dtype")
+        p.conv, p.taps = conv.data_ptr(), conv.shape[1]
+        if p.taps > 1:
+            tail = cache.tail
+            if tail is None or tail.dtype != y.dtype or tuple(tail.shape[1:]) != (p.taps - 1, c) or tail.shape[0] <= max(batch.slot) or not tail.is_contiguous():
+                raise ValueError("recurrent_prepare: the cache's tails do not fit the convolution or the step's slots")
+            p.tail = tail.data_ptr()
+    p.decay_bias, p.decay_rate = _f32(decay_bias, "decay_bias").data_ptr(), _f32(decay_rate, "decay_rate").data_ptr()
+    p.seq, p.tok, p.out, p.out_stride, p.T = batch.seq.data_ptr(), batch.tok.data_ptr(), out.data_ptr(), out.stride(0), t
+    p.H, p.G, p.dk, p.dv = lay.heads, lay.groups, lay.dk, lay.dv
+    p.off_q, p.off_k, p.off_v, p.off_beta = lay.off_q, lay.off_k, lay.off_v, lay.off_beta
+    p.unit, p.sign, p.q_scale, p.act = int(bool(unit)), float(sign), float(q_scale), act
+    _lib.check_mixers(_lib.mixers().gbxm_recurrent_prepare(ctypes.byref(p), _stream(y.device)))
+    return out
+
+
+def conv_tail_update(y: torch.Tensor, channels: int, cache, batch) -> None:
+    act = _act(y, "y")
+    tail = cache.tail
+    if y.stride(1) != 1 or y.shape[1] < channels or tail.dtype != y.dtype or tuple(tail.shape[1:]) != (cache.taps - 1, channels) or tail.shape[0] <= max(batch.slot):
+        raise ValueError("conv_tail_update: the cache's tails do not fit the rows or the step's slots")
+    _lib.check_mixers(_lib.mixers().gbxm_conv_tail_update(y.data_ptr(), y.stride(0), tail.data_ptr(), batch.seq.data_ptr(), len(batch.slot), channels,
+                                                         cache.taps, act, _stream(y.device)))
+
+
+def decayed_state_scan(r: torch.Tensor, lay, cache, batch, delta: bool) -> torch.Tensor:
+    _f32(r, "r")
+    state = cache.state
+    if not r.is_cuda or r.shape != (batch.total, lay.out_width) or (delta and lay.off_beta < 0):
+        raise ValueError("decayed_state_scan: prepared rows do not fit the step")
+    if state is None or state.dtype != torch.float32 or tuple(state.shape[1:]) != (lay.heads, lay.dv, lay.dk) or state.shape[0] <= max(batch.slot) or not state.is_contiguous():
+        raise ValueError("decayed_state_scan: the cache's states do not fit the mixer or the step's slots")
+    out = torch.empty((batch.total, lay.nv), dtype=torch.float32, device=r.device)
+    _lib.check_mixers(_lib.mixers().gbxm_state_scan(r.data_ptr(), r.stride(0), state.data_ptr(), out.data_ptr(), batch.seq.data_ptr(), len(batch.slot),
+                                                   lay.heads, lay.groups, lay.dk, lay.dv, int(bool(delta)), _stream(r.device)))
+    return out
+
+
+def head_norm_gate(o: torch.Tensor, gate: torch.Tensor, weight: torch.Tensor, heads: int, eps: float, kind: int) -> torch.Tensor:
+    act = _act(gate, "gate")
+    _f32(o, "o")
+    t, n = o.shape
+    if gate.shape != (t, n) or gate.stride(1) != 1 or n % heads or weight.numel() != n // heads:
+        raise ValueError("head_norm_gate: read-outs, gate and weight do not fit")
+    out = torch.empty((t, n), dtype=gate.dtype, device=o.device)
+    _lib.check_mixers(_lib.mixers().gbxm_head_norm_gate(o.data_ptr(), gate.data_ptr(), gate.stride(0), _f32(weight, "weight").data_ptr(), out.data_ptr(),
+                                                       t, heads, n // heads, float(eps), int(kind), act, _stream(o.device)))
     return out

@@ -136,6 +136,67 @@ typedef struct {
 int gbxm_sink_attention(const gbxm_sink_attn_args* a, void* stream);
 int gbxm_sink_attention_tiled(int32_t dk, int32_t dv, int32_t act, int32_t decode_only);
 
+/* ---- several residual streams, layer norm, gated activations, grouped sigmoid router (gbx-lm_amd/models/residual.py:hyper_step_,
+ * models/feed_forward.py:glu_, models/switch_layers.py) ---- */
+
+/* One sublayer boundary over streams X fp32 [T][S][width], in place, one workgroup per row:
+ *   if y:  z = y[t] (top == 1) or sum_k y_mix[t][k] y[t][k];   X_j <- sum_i mix[i][j] X_i + write[j] z   (all j from the old X)
+ *   u = sum_i read[i] X_i   (read null: plain sum)
+ *   norm_w: h = (u - mean) / sqrt(var + eps) * norm_w + norm_b in the activation dtype (var = mean of squared deviations), else
+ *   out_u = u (fp32).  S <= 8. */
+int gbxm_hyper_step(float* X, const void* y, const float* y_mix, const float* mix, const float* write, const float* read, const float* norm_w,
+                    const float* norm_b, void* h, float* out_u, int64_t T, int32_t S, int32_t width, int32_t top, float eps, int32_t act,
+                    void* stream);
+/* out[t][f] = act(gu[t][f], gu[t][F + f]) in fp32, rows of 2F in, F out (unit inner strides, row strides in elements).
+ * kind 1: g sigmoid(g) u;  kind 2: g' = min(g, limit), u' = clamp(u, -limit, limit), g' sigmoid(alpha g') (u' + 1). */
+#define GBXM_GLU_SILU 1
+#define GBXM_GLU_CLAMPED_SWISH 2
+int gbxm_glu(const void* gu, int64_t gu_stride, void* out, int64_t T, int32_t F, int32_t kind, float limit, float alpha, int32_t act, void* stream);
+/* Router decisions from fp32 logits [T][E]: s = sigmoid(logit), choice score c = s + correction; with n_groups > 0 the experts form
+ * n_groups equal groups of neighbours, a group's score is the sum of its two largest c, and only experts of the keep_groups best
+ * groups can be chosen; the `top` largest c are chosen (ties: lower index); weight = s (divided by the chosen sum + 1e-20 if
+ * renorm) * scale. */
+int gbxm_route_sigmoid_groups(const float* logits, const float* correction, int32_t* idx, float* weight, int64_t T, int32_t E, int32_t top,
+                              int32_t n_groups, int32_t keep_groups, int32_t renorm, float scale, void* stream);
+/* gbxm_expert_glu with the expert's activation as a parameter (GBXM_GLU_*, alpha = 1.702 for kind 2). */
+int gbxm_expert_glu_act(const void* h, const void* gate_up, const void* down, const int32_t* idx, void* y, int64_t T, int32_t K, int32_t F,
+                        int32_t E, int32_t top, int32_t act, int32_t kind, float limit, void* ws, size_t ws_bytes, void* stream);
+
+/* ---- recurrent mixers: a decayed matrix state per head (gbx-lm_amd/models/recurrent_mixers.py) ---- */
+
+/* Row preparation, everything in fp32.  y rows hold q (G*dk) | k (G*dk) | v (H*dv) at off_q / off_k / off_v and optionally beta (H) at
+ * off_beta (< 0: none); `a` rows [T][H*dk] are the decay projection.  With conv (rows [2 G dk + H dv][taps], q | k | v must be adjacent
+ * from off_q on): c[t] = silu(sum_j conv[c][j] in[t - (taps-1) + j]), inputs before the step from tail [slots][taps-1][C] (oldest
+ * first), zeros before the sequence.  unit: q, k heads / sqrt(sum sq + 1e-6).  out row: q * q_scale | k | v | decay | beta with
+ * decay = exp(-rate[h] * softplus(sign * (a + bias))), beta = sigmoid(.). */
+typedef struct {
+  const void* y;    int64_t y_stride;
+  const void* a;    int64_t a_stride;
+  const void* conv;             /* activation dtype, or null */
+  const void* tail;             /* activation dtype [slots][taps-1][C] */
+  const float* decay_bias;      /* [H*dk] */
+  const float* decay_rate;      /* [H] */
+  const int32_t* seq;           /* [B][4] */
+  const int32_t* tok;           /* [T][2] */
+  float* out;       int64_t out_stride;
+  int64_t T;
+  int32_t H, G, dk, dv, off_q, off_k, off_v, off_beta, taps, unit;
+  float sign, q_scale;
+  int32_t act;
+} gbxm_recurrent_prep_args;
+int gbxm_recurrent_prepare(const gbxm_recurrent_prep_args* a, void* stream);
+/* tail[slot] <- the last taps-1 inputs (channels [0, C) of y) of every sequence of the step; older ones shift out. */
+int gbxm_conv_tail_update(const void* y, int64_t y_stride, void* tail, const int32_t* seq, int32_t B, int32_t C, int32_t taps, int32_t act,
+                          void* stream);
+/* The scan over each sequence's new rows.  r: rows of gbxm_recurrent_prepare; state fp32 [slots][H][dv][dk] (read unless the sequence
+ * starts at position 0, written back); out fp32 [T][H*dv].  Per token: S <- diag(decay) S; delta: u = beta (v - S^T k) else u = v;
+ * S <- S + k u^T; o = S^T q.  dk <= 256. */
+int gbxm_state_scan(const float* r, int64_t r_stride, float* state, float* out, const int32_t* seq, int32_t B, int32_t H, int32_t G,
+                    int32_t dk, int32_t dv, int32_t delta, void* stream);
+/* out[t][h][c] = o[t][h][c] / sqrt(mean_c o^2 + eps) * w[c] * gate(g[t][h][c]); gate kind 1 silu, 2 sigmoid; o fp32, g / out activation dtype. */
+int gbxm_head_norm_gate(const float* o, const void* gate, int64_t gate_stride, const float* w, void* out, int64_t T, int32_t H, int32_t dv,
+                        float eps, int32_t kind, int32_t act, void* stream);
+
 #ifdef __cplusplus
 }
 #endif
