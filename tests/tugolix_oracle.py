@@ -217,3 +217,124 @@ def forward(cfg, weights, tokens):
         after.append(X.sum(1))
     logits = layer_norm(X.sum(1), w["final.norm"], w["final.norm.b"], eps) @ w["head"].T * cfg.get("logit_scale", 1.0)
     return logits, torch.stack(after)
+
+
+# ------------------------------------------------------------------------------------------------ configurations and checkpoints
+def gla_layer(heads, dim, vdim, tau, mlp=None):
+    return {"type": "gla", "mixer": {"heads": heads, "dim": dim, "vdim": vdim, "tau": tau}, "mlp": mlp}
+
+
+def delta_layer(heads, kv_heads, dim, vdim, conv, mlp=None):
+    return {"type": "channel_delta", "mixer": {"heads": heads, "kv_heads": kv_heads, "dim": dim, "vdim": vdim, "conv": conv}, "mlp": mlp}
+
+
+def latent_layer(heads, dim, vdim, kv_rank, scale=None, kv_from=None, mlp=None):
+    m = {"heads": heads, "dim": dim, "vdim": vdim, "kv_rank": kv_rank, "scale": scale if scale is not None else dim ** -0.5}
+    if kv_from is not None:
+        m["kv_from"] = kv_from
+    return {"type": "latent_attention", "mixer": m, "mlp": mlp}
+
+
+def dense(ff):
+    return {"kind": "dense", "ff": ff}
+
+
+def moe(experts, top, ff, limit=1.0, groups=None, scale=1.0):
+    r = {"experts": experts, "top": top, "scale": scale}
+    if groups:
+        r["groups"] = {"count": groups[0], "keep": groups[1]}
+    return {"kind": "moe", "expert": {"ff": ff, "limit": limit}, "router": r}
+
+
+def make_config(layers, vocab=61, width=64, eps=1e-5, streams=3, logit_scale=1.0):
+    cfg = {"architecture": "Tugolix", "vocab": vocab, "width": width, "layers": layers, "norm": {"eps": eps}, "logit_scale": logit_scale}
+    if streams:
+        cfg["streams"] = streams
+    return cfg
+
+
+def make_weights(cfg, seed=0, decay_rank=6, gate_rank=5, steady_router=False):
+    """``steady_router``: the corrections lie 0.3 apart and the router matrix is small, so that no rounding of a token's input can
+    change which experts it gets (for whole models in bfloat16, where a changed choice in one layer would change the recurrent state
+    of every later token)."""
+    gen = torch.Generator().manual_seed(seed)
+    W, s = cfg["width"], cfg.get("streams")
+    bf = torch.bfloat16
+
+    def mat(o, i, scale=1.0):
+        return (torch.randn((o, i), generator=gen) * scale / math.sqrt(i)).to(bf)
+
+    def vec(n, lo, hi):
+        return (torch.rand((n,), generator=gen) * (hi - lo) + lo).to(bf)
+
+    w = {"embed": torch.randn((cfg["vocab"], W), generator=gen).to(bf), "final.norm": vec(W, 0.5, 1.5), "final.norm.b": vec(W, -0.3, 0.3),
+         "head": mat(cfg["vocab"], W)}
+    for i, layer in enumerate(cfg["layers"]):
+        p, m, kind = f"l{i}.", layer["mixer"], layer["type"]
+        for q in (1, 2) if layer.get("mlp") is not None else (1,):
+            w[p + f"norm{q}"], w[p + f"norm{q}.b"] = vec(W, 0.5, 1.5), vec(W, -0.3, 0.3)
+            if s:
+                w[p + f"hc{q}.in"], w[p + f"hc{q}.out"] = vec(s, 0.1, 0.7), vec(s, 0.7, 1.3)
+                w[p + f"hc{q}.mix"] = (torch.eye(s) * 0.8 + torch.randn((s, s), generator=gen) * 0.2).to(bf)
+        H, d, dv = m["heads"], m["dim"], m["vdim"]
+        x = p + "mix."
+        if kind == "gla":
+            w[x + "q"], w[x + "k"], w[x + "v"], w[x + "g"] = mat(H * d, W), mat(H * d, W), mat(H * dv, W), mat(H * dv, W)
+            w[x + "a1"], w[x + "a2"], w[x + "a2.b"] = mat(decay_rank, W), mat(H * d, decay_rank, 2.0), vec(H * d, -1.0, 5.0)
+            w[x + "norm"], w[x + "o"] = vec(dv, 0.5, 1.5), mat(W, H * dv)
+        elif kind == "channel_delta":
+            G, taps = m["kv_heads"], m["conv"]
+            w[x + "q"], w[x + "k"], w[x + "v"] = mat(G * d, W), mat(G * d, W), mat(H * dv, W)
+            for nm, n in (("q", G * d), ("k", G * d), ("v", H * dv)):
+                w[x + nm + ".conv"] = (torch.randn((n, taps), generator=gen) * 0.7 + 0.25).to(bf)
+            w[x + "b"], w[x + "A_log"], w[x + "dt_bias"] = mat(H, W, 2.0), vec(H, -4.0, 0.0), vec(H * d, -4.0, -1.0)
+            w[x + "a1"], w[x + "a2"] = mat(decay_rank, W), mat(H * d, decay_rank, 2.0)
+            w[x + "g1"], w[x + "g2"] = mat(gate_rank, W), mat(H * dv, gate_rank, 2.0)
+            w[x + "norm"], w[x + "o"] = vec(dv, 0.5, 1.5), mat(W, H * dv)
+        else:
+            R = m["kv_rank"]
+            w[x + "q"], w[x + "uk"], w[x + "uv"], w[x + "o"] = mat(H * d, W), mat(H * d, R), mat(H * dv, R), mat(W, H * dv)
+            if "kv_from" not in m:
+                w[x + "dkv"], w[x + "dkv.norm"] = mat(R, W, 2.0), vec(R, 0.5, 1.5)
+        ff = layer.get("mlp")
+        f = p + "mlp."
+        if ff is not None and ff["kind"] == "dense":
+            n = ff["ff"]
+            w[f + "gate"], w[f + "up"], w[f + "down"] = mat(n, W), mat(n, W), mat(W, n)
+            w[f + "gate.b"], w[f + "up.b"], w[f + "down.b"] = vec(n, -0.3, 0.3), vec(n, -0.3, 0.3), vec(W, -0.3, 0.3)
+        elif ff is not None:
+            n, E = ff["expert"]["ff"], ff["router"]["experts"]
+            w[f + "router"], w[f + "correction"] = mat(E, W, 1.5), vec(E, -1.5, -0.5)
+            if steady_router:
+                w[f + "router"] = mat(E, W, 0.1)
+                w[f + "correction"] = (torch.randperm(E, generator=gen).float() * 0.3 - 2.0).to(bf)
+            for e in range(E):
+                w[f + f"e{e}.gate"], w[f + f"e{e}.up"], w[f + f"e{e}.down"] = mat(n, W, 1.5), mat(n, W, 1.5), mat(W, n)
+    return w
+
+
+def save_checkpoint(folder, cfg, weights):
+    from safetensors.torch import save_file
+    os.makedirs(folder, exist_ok=True)
+    with open(os.path.join(folder, "config.json"), "w") as f:
+        json.dump(cfg, f)
+    save_file({k: v.contiguous() for k, v in weights.items()}, os.path.join(folder, "model.safetensors"))
+    return folder
+
+
+def row_errors(got, want):
+    """Root mean square of the difference over that of the reference, per row."""
+    got, want = got.to(F64).cpu(), want.to(F64).cpu()
+    return (got - want).pow(2).mean(-1).sqrt() / want.pow(2).mean(-1).sqrt().clamp_min(1e-12)
+
+
+def rel_err(got, want):
+    """The worst row's error."""
+    return float(row_errors(got, want).max())
+
+
+def rel_err_most(got, want, share=0.9):
+    """The error that ``share`` of the rows stay under.  For whole models in bfloat16: a router whose two candidates lie closer than
+    the rounding of its input may choose the other one, and that row then differs by a whole expert."""
+    e = row_errors(got, want).flatten().sort().values
+    return float(e[min(int(math.ceil(share * e.numel())) - 1, e.numel() - 1)])
