@@ -254,9 +254,9 @@ def make_config(layers, vocab=61, width=64, eps=1e-5, streams=3, logit_scale=1.0
 
 
 def make_weights(cfg, seed=0, decay_rank=6, gate_rank=5, steady_router=False):
-    """``steady_router``: the corrections lie 0.3 apart and the router matrix is small, so that no rounding of a token's input can
-    change which experts it gets (for whole models in bfloat16, where a changed choice in one layer would change the recurrent state
-    of every later token)."""
+    """``steady_router``: the corrections are distinct powers of two (times -1/8: all sums of two differ by 1/8 or more) and the
+    router matrix is small, so that no rounding of a token's input can change its groups or experts (for whole models in bfloat16,
+    where a changed choice in one layer would change the recurrent state of every later token)."""
     gen = torch.Generator().manual_seed(seed)
     W, s = cfg["width"], cfg.get("streams")
     bf = torch.bfloat16
@@ -307,7 +307,7 @@ def make_weights(cfg, seed=0, decay_rank=6, gate_rank=5, steady_router=False):
             w[f + "router"], w[f + "correction"] = mat(E, W, 1.5), vec(E, -1.5, -0.5)
             if steady_router:
                 w[f + "router"] = mat(E, W, 0.1)
-                w[f + "correction"] = (torch.randperm(E, generator=gen).float() * 0.3 - 2.0).to(bf)
+                w[f + "correction"] = (-0.125 * 2.0 ** torch.randperm(E, generator=gen).float()).to(bf)
             for e in range(E):
                 w[f + f"e{e}.gate"], w[f + f"e{e}.up"], w[f + f"e{e}.down"] = mat(n, W, 1.5), mat(n, W, 1.5), mat(W, n)
     return w
