@@ -626,12 +626,85 @@ def radenex_bench(args):
     print(json.dumps({"metric": "radenex_throughput", "unit": "tokens/s", "dtype": "bf16", "data": "synthetic", "sizes": out}))
 
 
+TUGOLIX_SIZES = {
+    # name: Tugolix geometry (layers: channel-wise delta rule, gated linear attention, latent attention, latent attention over the same
+    # rows; dense feed-forward in the first layer, routed experts in the others) and, from it, the Revitar (the closest existing model:
+    # dense bf16 decoder over ragged steps with routed experts) of equal width, experts and layer count
+    "small": dict(width=1024, delta=dict(heads=8, kv_heads=4, dim=64, vdim=128, conv=4), gla=dict(heads=4, dim=128, vdim=256, tau=16.0),
+                  latent=dict(heads=8, dim=64, vdim=64, kv_rank=256), ff=4096, moe=dict(experts=32, top=4, ff=512, groups=(8, 4)), pattern="dgls"),
+    "a3b-like": dict(width=2048, delta=dict(heads=32, kv_heads=16, dim=128, vdim=128, conv=4), gla=dict(heads=8, dim=128, vdim=256, tau=16.0),
+                     latent=dict(heads=16, dim=128, vdim=128, kv_rank=512), ff=8192, moe=dict(experts=128, top=8, ff=768, groups=(8, 4)),
+                     pattern="dgls"),
+    "recurrent": dict(width=2048, delta=dict(heads=16, kv_heads=16, dim=128, vdim=128, conv=4), gla=dict(heads=8, dim=128, vdim=256, tau=16.0),
+                      latent=dict(heads=16, dim=128, vdim=128, kv_rank=512), ff=8192, moe=dict(experts=64, top=4, ff=1024, groups=(4, 2)),
+                      pattern="dgdg"),
+}
+
+
+def tugolix_bench(args):
+    """``--design tugolix``: prefill and decode throughput of Tugolix at layer sizes of real models (random weights, bf16), beside
+    Revitar of equal width, layer count and routed experts, its attention with the delta layers' head geometry.  One JSON line; the
+    default workload of this file is untouched."""
+    from gbx_lm_amd import synthetic as S
+    from gbx_lm_amd.batching import BatchScheduler
+    dev = torch.device("cuda", 0)
+    torch.cuda.set_device(dev)
+
+    def clock(fn, reps):
+        fn()
+        torch.cuda.synchronize()
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record()
+        for _ in range(reps):
+            fn()
+        e1.record()
+        torch.cuda.synchronize()
+        return e0.elapsed_time(e1) / reps
+
+    def legs(model, vocab, tag, res):
+        toks = lambda n, o=0: [(o + i * 7919) % vocab for i in range(n)]
+        for T in (512, 4096):
+            def prefill():
+                eng = BatchScheduler(model)
+                eng.step([("p", toks(T))])
+            res[f"{tag}prefill_T{T}_tok_s"] = round(T / clock(prefill, 3) * 1e3)
+        for B, ctx in ((1, 2048), (32, 256)):
+            eng = BatchScheduler(model)
+            eng.step([(i, toks(ctx, i)) for i in range(B)])
+            state = {"t": 0}
+            def decode():
+                state["t"] += 1
+                eng.step([(i, [(state["t"] * 31 + i) % vocab]) for i in range(B)])
+            res[f"{tag}decode_B{B}_ctx{ctx}_tok_s"] = round(B / clock(decode, 64) * 1e3)
+            del eng
+        print(tag or "tugolix", res, file=sys.stderr, flush=True)
+
+    out = {}
+    for name in args.sizes.split(","):
+        g = TUGOLIX_SIZES[name]
+        res = {"geometry": g}
+        cfg = S.tugolix_config(**g)
+        model = S.build_tugolix(cfg, device=dev, seed=0)
+        legs(model, cfg["vocab"], "", res)
+        del model
+        torch.cuda.empty_cache()
+        d, m = g["delta"], g["moe"]
+        rm = S.build_revitar(S.revitar_config(width=g["width"], heads=d["heads"], kv_heads=d["kv_heads"], dim=d["dim"], vdim=d["vdim"], window=4096,
+                                              experts=m["experts"], top=m["top"], ff=m["ff"], n_layers=len(g["pattern"]), vocab=cfg["vocab"]),
+                             device=dev, seed=0)
+        legs(rm, cfg["vocab"], "revitar_", res)
+        del rm
+        torch.cuda.empty_cache()
+        out[name] = res
+    print(json.dumps({"metric": "tugolix_throughput", "unit": "tokens/s", "dtype": "bf16", "data": "synthetic", "sizes": out}))
+
+
 def main():
     ap = argparse.ArgumentParser()
-    ap.add_argument("--design", default=None, choices=["revitar", "radenex"], help="side benchmark of one model design beside the closest existing "
+    ap.add_argument("--design", default=None, choices=["revitar", "radenex", "tugolix"], help="side benchmark of one model design beside the closest existing "
                     "family at equal size (own JSON line; the default workload and its output are unchanged)")
     ap.add_argument("--sizes", default=None, help="--design: comma-separated names of REVITAR_SIZES (default small,a3b-like) / RADENEX_SIZES "
-                    "(default small,lite-like)")
+                    "(default small,lite-like) / TUGOLIX_SIZES (default small,a3b-like)")
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=512, help="timed decode steps (default: > 0.5 s of GPU time, so that a coarse GPU-busy sampler sees the run)")
     ap.add_argument("--warmup", type=int, default=8)
@@ -650,8 +723,8 @@ def main():
     if args.design is not None:
         if not torch.cuda.is_available():
             raise SystemExit("bench.py needs an MI355X")
-        args.sizes = args.sizes or {"revitar": "small,a3b-like", "radenex": "small,lite-like"}[args.design]
-        return revitar_bench(args) if args.design == "revitar" else radenex_bench(args)
+        args.sizes = args.sizes or {"revitar": "small,a3b-like", "radenex": "small,lite-like", "tugolix": "small,a3b-like"}[args.design]
+        return {"revitar": revitar_bench, "radenex": radenex_bench, "tugolix": tugolix_bench}[args.design](args)
     if args.gpus > 1 and "WORLD_SIZE" not in os.environ:
         spawn_ranks(args.gpus)                                     # never returns; nothing has touched the GPU yet
     world = int(os.environ.get("WORLD_SIZE", "1"))

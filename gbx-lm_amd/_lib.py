@@ -393,7 +393,7 @@ def mixers() -> ctypes.CDLL:
         L.gbxm_expert_glu_act.argtypes = [p, p, p, p, p, i64, i32, i32, i32, i32, i32, i32, f32, p, sz, p]
         L.gbxm_recurrent_prepare.argtypes = [ctypes.POINTER(RecurrentPrepArgs), p]
         L.gbxm_conv_tail_update.argtypes = [p, i64, p, p, i32, i32, i32, i32, p]
-        L.gbxm_state_scan.argtypes = [p, i64, p, p, p, i32, i32, i32, i32, i32, i32, p]
+        L.gbxm_state_scan.argtypes = [p, i64, p, p, p, i32, i64, i32, i32, i32, i32, i32, p]
         L.gbxm_head_norm_gate.argtypes = [p, p, i64, p, p, i64, i32, i32, f32, i32, i32, p]
         _mlib = L
     return _mlib

@@ -4,10 +4,11 @@
 //                           exp(-rate_h softplus(sign (a + bias))) and beta = sigmoid(b), all in fp32, into one fp32 row.
 //   conv_tail_kernel        the last taps-1 convolution inputs of every sequence into its slot.
 //   state_scan_kernel<R>    the scan.  The columns of a head's state (one per value channel) never meet: a wave takes four columns, 16
-//                           lanes per column, a lane holds R neighbouring key channels of its column in registers; per token the two
-//                           dot products over key channels are R multiply-adds and four cross-lane adds inside a 16-lane row (all 16
-//                           lanes end with the same bits).  The next token's operands are fetched while the current one is computed.
-//                           Sums run in a fixed order: a sequence's result does not depend on what else is in the step.
+//                           lanes per column, a lane holds R key channels of its column in registers; per token the two dot products
+//                           over key channels are R multiply-adds and four cross-lane adds inside a 16-lane row (all 16 lanes end
+//                           with the same bits).  Operands come through LDS in chunks of tokens, the next chunk fetched while the
+//                           current one is computed.  Sums run in a fixed order: a sequence's result does not depend on what else is
+//                           in the step, nor on how many columns a workgroup takes.
 //   head_norm_gate_kernel   per-head RMS norm of the read-out, weight and gate, one wave per (row, head).
 #include "mixers_common.h"
 
@@ -98,67 +99,96 @@ __device__ __forceinline__ float row16_sum(float v) {
   return v;
 }
 
-template <int R, bool DELTA>
-__global__ __launch_bounds__(64) void state_scan_kernel(const float* __restrict__ r, int64_t r_stride, float* __restrict__ state,
-                                                       float* __restrict__ out, const int* __restrict__ seq, int H, int G, int dk, int dv) {
+// NW waves per workgroup = 4 NW columns of one (sequence, head).  The operands of CH tokens (q | k | decay padded to 16 R channels, the
+// workgroup's value columns, beta) are staged in LDS, shared by the waves, two buffers: the next chunk is fetched into registers before
+// the current one is computed and parked in the other buffer afterwards, one barrier per chunk.  Lane ks of a 16-lane row owns the key
+// channels ks, ks + 16, ...: LDS reads and the state's loads and stores are contiguous over the row.
+template <int R, bool DELTA, int NW>
+__global__ __launch_bounds__(64 * NW) void state_scan_kernel(const float* __restrict__ r, int64_t r_stride, float* __restrict__ state,
+                                                            float* __restrict__ out, const int* __restrict__ seq, int H, int G, int dk, int dv) {
+  constexpr int DKP = 16 * R, NCOL = 4 * NW, ROW = 3 * DKP + NCOL + 1, NTH = 64 * NW;
+  constexpr int CH = (R <= 4 ? 32 : (R <= 8 ? 16 : 8)) * NW / 4;
+  constexpr int PF = (CH * ROW + NTH - 1) / NTH;
+  __shared__ float buf[2][CH * ROW];
   const int b = blockIdx.z, h = blockIdx.y;
-  const int lane = threadIdx.x, ks = lane & 15;
-  const int col = blockIdx.x * 4 + (lane >> 4);
+  const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63, ks = lane & 15;
+  const int col0 = blockIdx.x * NCOL, lcol = wave * 4 + (lane >> 4), col = col0 + lcol;
   const int slot = seq[4 * b], pos0 = seq[4 * b + 1], n = seq[4 * b + 2], row0 = seq[4 * b + 3];
   const bool col_ok = col < dv;
   const int colc = col_ok ? col : dv - 1;
-  const int c0 = ks * R;
   const int nq = G * dk, nv = H * dv;
   const int g = h / (H / G);
-  float* sp = state + ((static_cast<int64_t>(slot) * H + h) * dv + colc) * dk + c0;
+  float* sp = state + ((static_cast<int64_t>(slot) * H + h) * dv + colc) * dk + ks;
   float S[R];
 #pragma unroll
-  for (int i = 0; i < R; ++i) S[i] = (pos0 > 0 && c0 + i < dk) ? sp[i] : 0.f;
+  for (int i = 0; i < R; ++i) S[i] = (pos0 > 0 && ks + 16 * i < dk) ? sp[16 * i] : 0.f;
   const float* base = r + static_cast<int64_t>(row0) * r_stride;
-  const int oq = g * dk + c0, ok = nq + g * dk + c0, ov = 2 * nq + h * dv + colc, og = 2 * nq + nv + h * dk + c0, ob = 2 * nq + nv + H * dk + h;
-  float q[R], k[R], d[R], v, beta = 1.f;
-  auto fetch = [&](const float* rp, float* fq, float* fk, float* fd, float& fv, float& fb) {
+  const int oq = g * dk, ok = nq + g * dk, ov = 2 * nq + h * dv, og = 2 * nq + nv + h * dk, ob = 2 * nq + nv + H * dk + h;
+  float pf[PF];
+  auto fetch = [&](int t0) {
 #pragma unroll
-    for (int i = 0; i < R; ++i) {
-      const bool in = c0 + i < dk;
-      fq[i] = in ? rp[oq + i] : 0.f;
-      fk[i] = in ? rp[ok + i] : 0.f;
-      fd[i] = in ? rp[og + i] : 1.f;
+    for (int i = 0; i < PF; ++i) {
+      const int idx = threadIdx.x + i * NTH;
+      const int tt = idx / ROW, j = idx - tt * ROW;
+      float val = 0.f;
+      if (idx < CH * ROW && t0 + tt < n) {
+        const float* rp = base + static_cast<int64_t>(t0 + tt) * r_stride;
+        if (j < DKP) val = j < dk ? rp[oq + j] : 0.f;
+        else if (j < 2 * DKP) val = j - DKP < dk ? rp[ok + j - DKP] : 0.f;
+        else if (j < 3 * DKP) val = j - 2 * DKP < dk ? rp[og + j - 2 * DKP] : 1.f;
+        else if (j < 3 * DKP + NCOL) val = col0 + j - 3 * DKP < dv ? rp[ov + col0 + j - 3 * DKP] : 0.f;
+        else val = DELTA ? rp[ob] : 1.f;
+      }
+      pf[i] = val;
     }
-    fv = rp[ov];
-    if constexpr (DELTA) fb = rp[ob];
   };
-  fetch(base, q, k, d, v, beta);
+  auto park = [&](float* dst) {
+#pragma unroll
+    for (int i = 0; i < PF; ++i) {
+      const int idx = threadIdx.x + i * NTH;
+      if (idx < CH * ROW) dst[idx] = pf[i];
+    }
+  };
+  fetch(0);
+  park(buf[0]);
+  __syncthreads();
   float* op = out + static_cast<int64_t>(row0) * nv + h * dv + colc;
-  for (int t = 0; t < n; ++t) {
-    float nq_[R], nk_[R], nd_[R], nv_ = 0.f, nb_ = 1.f;
-    const bool more = t + 1 < n;
-    if (more) fetch(base + static_cast<int64_t>(t + 1) * r_stride, nq_, nk_, nd_, nv_, nb_);
-    float u = v;
+  int which = 0;
+  for (int t0 = 0; t0 < n; t0 += CH, which ^= 1) {
+    const bool more = t0 + CH < n;
+    if (more) fetch(t0 + CH);
+    const float* cur = buf[which];
+    const int cn = min(CH, n - t0);
+#pragma unroll 2
+    for (int tt = 0; tt < cn; ++tt) {
+      const float* row = cur + tt * ROW;
+      float q[R], k[R];
 #pragma unroll
-    for (int i = 0; i < R; ++i) S[i] *= d[i];
-    if constexpr (DELTA) {
-      float dot = 0.f;
+      for (int i = 0; i < R; ++i) {
+        q[i] = row[ks + 16 * i];
+        k[i] = row[DKP + ks + 16 * i];
+        S[i] *= row[2 * DKP + ks + 16 * i];
+      }
+      float u = row[3 * DKP + lcol];
+      if constexpr (DELTA) {
+        float dot = 0.f;
 #pragma unroll
-      for (int i = 0; i < R; ++i) dot += k[i] * S[i];
-      u = beta * (v - row16_sum(dot));
+        for (int i = 0; i < R; ++i) dot += k[i] * S[i];
+        u = row[3 * DKP + NCOL] * (u - row16_sum(dot));
+      }
+      float o = 0.f;
+#pragma unroll
+      for (int i = 0; i < R; ++i) { S[i] += k[i] * u; o += q[i] * S[i]; }
+      o = row16_sum(o);
+      if (ks == 0 && col_ok) op[static_cast<int64_t>(t0 + tt) * nv] = o;
     }
-    float o = 0.f;
-#pragma unroll
-    for (int i = 0; i < R; ++i) { S[i] += k[i] * u; o += q[i] * S[i]; }
-    o = row16_sum(o);
-    if (ks == 0 && col_ok) op[static_cast<int64_t>(t) * nv] = o;
-    if (more) {
-#pragma unroll
-      for (int i = 0; i < R; ++i) { q[i] = nq_[i]; k[i] = nk_[i]; d[i] = nd_[i]; }
-      v = nv_;
-      beta = nb_;
-    }
+    if (more) park(buf[which ^ 1]);
+    __syncthreads();
   }
   if (col_ok) {
 #pragma unroll
     for (int i = 0; i < R; ++i)
-      if (c0 + i < dk) sp[i] = S[i];
+      if (ks + 16 * i < dk) sp[16 * i] = S[i];
   }
 }
 
@@ -182,10 +212,11 @@ __global__ __launch_bounds__(NT) void head_norm_gate_kernel(const float* __restr
   }
 }
 
-template <bool DELTA>
-int launch_scan(int R, dim3 grid, hipStream_t s, const float* r, int64_t r_stride, float* state, float* out, const int32_t* seq, int H, int G, int dk,
+template <bool DELTA, int NW>
+int launch_scan(int R, int B, hipStream_t s, const float* r, int64_t r_stride, float* state, float* out, const int32_t* seq, int H, int G, int dk,
                 int dv) {
-#define GBXM_SCAN(N) state_scan_kernel<N, DELTA><<<grid, 64, 0, s>>>(r, r_stride, state, out, seq, H, G, dk, dv)
+  const dim3 grid((dv + 4 * NW - 1) / (4 * NW), H, B);
+#define GBXM_SCAN(N) state_scan_kernel<N, DELTA, NW><<<grid, 64 * NW, 0, s>>>(r, r_stride, state, out, seq, H, G, dk, dv)
   if (R <= 1) GBXM_SCAN(1);
   else if (R <= 2) GBXM_SCAN(2);
   else if (R <= 3) GBXM_SCAN(3);
@@ -236,8 +267,8 @@ int gbxm_conv_tail_update(const void* y, int64_t y_stride, void* tail, const int
   return after_launch("conv_tail_update");
 }
 
-int gbxm_state_scan(const float* r, int64_t r_stride, float* state, float* out, const int32_t* seq, int32_t B, int32_t H, int32_t G, int32_t dk,
-                    int32_t dv, int32_t delta, void* stream) {
+int gbxm_state_scan(const float* r, int64_t r_stride, float* state, float* out, const int32_t* seq, int32_t B, int64_t T_, int32_t H, int32_t G,
+                    int32_t dk, int32_t dv, int32_t delta, void* stream) {
   if (!r || !state || !out || !seq || B < 0 || H < 1 || G < 1 || H % G || dk < 1 || dv < 1 ||
       r_stride < 2 * G * dk + H * dv + H * dk + (delta ? H : 0))
     return fail(GBXM_ERR_INVALID, "state_scan: bad argument");
@@ -245,10 +276,14 @@ int gbxm_state_scan(const float* r, int64_t r_stride, float* state, float* out, 
   if (B == 0) return GBXM_OK;
   if (B > 65535 || H > 65535) return fail(GBXM_ERR_UNSUPPORTED, "state_scan: grid");
   hipStream_t s = static_cast<hipStream_t>(stream);
-  const dim3 grid((dv + 3) / 4, H, B);
   const int R = (dk + 15) / 16;
-  return delta ? launch_scan<true>(R, grid, s, r, r_stride, state, out, seq, H, G, dk, dv)
-               : launch_scan<false>(R, grid, s, r, r_stride, state, out, seq, H, G, dk, dv);
+  // long rows (prompts): 16 columns per workgroup share the staged operands; a few rows per sequence: 4 columns, four times the
+  // workgroups for the state's traffic.  A column's arithmetic is the same in both.
+  if (T_ >= 8 * static_cast<int64_t>(B))
+    return delta ? launch_scan<true, 4>(R, B, s, r, r_stride, state, out, seq, H, G, dk, dv)
+                 : launch_scan<false, 4>(R, B, s, r, r_stride, state, out, seq, H, G, dk, dv);
+  return delta ? launch_scan<true, 1>(R, B, s, r, r_stride, state, out, seq, H, G, dk, dv)
+               : launch_scan<false, 1>(R, B, s, r, r_stride, state, out, seq, H, G, dk, dv);
 }
 
 int gbxm_head_norm_gate(const float* o, const void* gate, int64_t gate_stride, const float* w, void* out, int64_t T_, int32_t H, int32_t dv,

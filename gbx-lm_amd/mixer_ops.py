@@ -408,7 +408,7 @@ def decayed_state_scan(r: torch.Tensor, lay, cache, batch, delta: bool) -> torch
         raise ValueError("decayed_state_scan: the cache's states do not fit the mixer or the step's slots")
     out = torch.empty((batch.total, lay.nv), dtype=torch.float32, device=r.device)
     _lib.check_mixers(_lib.mixers().gbxm_state_scan(r.data_ptr(), r.stride(0), state.data_ptr(), out.data_ptr(), batch.seq.data_ptr(), len(batch.slot),
-                                                   lay.heads, lay.groups, lay.dk, lay.dv, int(bool(delta)), _stream(r.device)))
+                                                   batch.total, lay.heads, lay.groups, lay.dk, lay.dv, int(bool(delta)), _stream(r.device)))
     return out
 
 

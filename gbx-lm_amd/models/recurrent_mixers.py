@@ -238,7 +238,7 @@ class ChannelDeltaRule(_RecurrentMixer):
 
     def fuse_weights(self, q, k, v, b, a1, g1):
         """The input projection from the checkpoint's matrices (all [out, in]), with the empty rows between the parts."""
-        w = torch.zeros((self.inp.out_features, q.shape[1]), dtype=q.dtype)
+        w = torch.zeros((self.inp.out_features, q.shape[1]), dtype=q.dtype, device=q.device)
         lay = self.layout
         for off, part in ((0, q), (lay.off_k, k), (lay.off_v, v), (lay.off_beta, b), (self.off_a1, a1), (self.off_g1, g1)):
             w[off:off + part.shape[0]] = part

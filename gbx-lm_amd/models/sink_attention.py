@@ -247,9 +247,9 @@ class LatentAttention(nn.Module):
     def fuse_weights(self, q, dkv, g, uk, uv):
         """The module's matrices from the checkpoint's (all [out, in]); ``dkv`` / ``g`` None for a mixer without them."""
         h, d, r, dv, rank = self.heads, self.dim, self.rot_dim, self.vdim, self.kv_rank
-        uk_pad = torch.cat([uk.view(h, d, rank), torch.zeros((h, r, rank), dtype=uk.dtype)], dim=1).reshape(h * (d + r), rank)
+        uk_pad = torch.cat([uk.view(h, d, rank), torch.zeros((h, r, rank), dtype=uk.dtype, device=uk.device)], dim=1).reshape(h * (d + r), rank)
         parts = [q] + ([dkv] if self.own_latent else []) + ([g] if self.gated else [])
-        pad = torch.zeros((self.inp.out_features - sum(p.shape[0] for p in parts), q.shape[1]), dtype=q.dtype)
+        pad = torch.zeros((self.inp.out_features - sum(p.shape[0] for p in parts), q.shape[1]), dtype=q.dtype, device=q.device)
         return {"inp.weight": torch.cat(parts + [pad]), "up.weight": torch.cat([uk_pad, uv]),
                 "uk_heads": uk.view(h, d, rank).contiguous(), "uv_heads_t": uv.view(h, dv, rank).transpose(1, 2).contiguous()}
 

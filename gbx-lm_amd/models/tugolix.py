@@ -205,7 +205,7 @@ class Model(RaggedStepModel):
             m = p + "mix."
             if kind == "gla":
                 parts = [weights[m + "q"], weights[m + "k"], weights[m + "v"], weights[m + "g"], weights[m + "a1"]]
-                pad = torch.zeros((mixer.inp.out_features - sum(x.shape[0] for x in parts), self.args.width), dtype=parts[0].dtype)
+                pad = torch.zeros((mixer.inp.out_features - sum(x.shape[0] for x in parts), self.args.width), dtype=parts[0].dtype, device=parts[0].device)
                 out[t + "mixer.inp.weight"] = torch.cat(parts + [pad])
                 out[t + "mixer.a2.weight"] = weights[m + "a2"]
                 out[t + "mixer.decay_bias"] = f32(weights[m + "a2.b"])

@@ -363,3 +363,105 @@ def build_radenex(config: Dict, device="cpu", seed: int = 0, act_dtype=torch.bfl
             m._buffers["uv_heads_t"] = up[h * (d + r):].view(h, dv, rank).transpose(1, 2).contiguous()
     model.eval()
     return model
+
+
+# ------------------------------------------------------------------------------------------------ Tugolix (several streams, recurrent and latent mixers)
+def tugolix_config(width: int, delta: Dict, gla: Dict, latent: Dict, ff: int, moe: Dict, pattern: str = "dgls", streams: int = 4,
+                   vocab: int = 32000) -> Dict:
+    """config.json of a Tugolix model: ``pattern`` names the layers in order ('d' channel-wise delta rule, 'g' gated linear attention,
+    'l' latent attention, 's' latent attention over the rows of the nearest 'l' before it); the first layer has the dense
+    feed-forward of ``ff`` channels, the others the routed one.  ``delta``: heads, kv_heads, dim, vdim, conv; ``gla``: heads, dim, vdim,
+    tau; ``latent``: heads, dim, vdim, kv_rank; ``moe``: experts, top, ff, groups (count, keep), limit, scale."""
+    routed = {"kind": "moe", "expert": {"ff": moe["ff"], "limit": moe.get("limit", 7.0)},
+              "router": {"experts": moe["experts"], "top": moe["top"], "scale": moe.get("scale", 2.5),
+                         "groups": {"count": moe["groups"][0], "keep": moe["groups"][1]}}}
+    layers, owner = [], None
+    for i, c in enumerate(pattern):
+        if c == "d":
+            layer = {"type": "channel_delta", "mixer": {k: delta[k] for k in ("heads", "kv_heads", "dim", "vdim", "conv")}}
+        elif c == "g":
+            layer = {"type": "gla", "mixer": {k: gla[k] for k in ("heads", "dim", "vdim", "tau")}}
+        else:
+            layer = {"type": "latent_attention", "mixer": dict({k: latent[k] for k in ("heads", "dim", "vdim", "kv_rank")}, scale=latent["dim"] ** -0.5)}
+            if c == "s":
+                if owner is None:
+                    raise ValueError("tugolix_config: 's' needs an 'l' before it")
+                layer["mixer"]["kv_from"] = owner
+            else:
+                owner = i
+        layer["mlp"] = {"kind": "dense", "ff": ff} if i == 0 else json.loads(json.dumps(routed))
+        layers.append(layer)
+    return {"architecture": "Tugolix", "vocab": vocab, "width": width, "norm": {"eps": 1e-6}, "streams": streams, "logit_scale": 1.0, "layers": layers}
+
+
+def tugolix_checkpoint(config: Dict, device="cpu", seed: int = 0, decay_rank: int = 64, gate_rank: int = 64, dtype=torch.bfloat16) -> Dict[str, torch.Tensor]:
+    """Random tensors in the design's checkpoint names with real shapes, generated directly on ``device``."""
+    device = torch.device(device)
+    gen = torch.Generator(device=device)
+    gen.manual_seed(seed)
+    W, s = config["width"], config.get("streams")
+
+    def mat(o, i, mult=1.0):
+        return (torch.randn((o, i), device=device, generator=gen) * (mult * i ** -0.5)).to(dtype)
+
+    def vec(n, lo, hi):
+        return (torch.rand((n,), device=device, generator=gen) * (hi - lo) + lo).to(dtype)
+
+    w = {"embed": torch.randn((config["vocab"], W), device=device, generator=gen).to(dtype), "final.norm": vec(W, 0.9, 1.1),
+         "final.norm.b": vec(W, -0.1, 0.1), "head": mat(config["vocab"], W)}
+    for i, layer in enumerate(config["layers"]):
+        p, m, kind = f"l{i}.", layer["mixer"], layer["type"]
+        for q in (1, 2) if layer.get("mlp") is not None else (1,):
+            w[p + f"norm{q}"], w[p + f"norm{q}.b"] = vec(W, 0.9, 1.1), vec(W, -0.1, 0.1)
+            if s:
+                w[p + f"hc{q}.in"], w[p + f"hc{q}.out"] = vec(s, 0.1, 0.6), vec(s, 0.8, 1.2)
+                w[p + f"hc{q}.mix"] = (torch.eye(s, device=device) * 0.9 + torch.randn((s, s), device=device, generator=gen) * 0.05).to(dtype)
+        H, d, dv, x = m["heads"], m["dim"], m["vdim"], p + "mix."
+        if kind == "gla":
+            w[x + "q"], w[x + "k"], w[x + "v"], w[x + "g"] = mat(H * d, W), mat(H * d, W), mat(H * dv, W), mat(H * dv, W)
+            w[x + "a1"], w[x + "a2"], w[x + "a2.b"] = mat(decay_rank, W), mat(H * d, decay_rank), vec(H * d, 0.0, 5.0)
+            w[x + "norm"], w[x + "o"] = vec(dv, 0.9, 1.1), mat(W, H * dv)
+        elif kind == "channel_delta":
+            G, taps = m["kv_heads"], m["conv"]
+            w[x + "q"], w[x + "k"], w[x + "v"] = mat(G * d, W), mat(G * d, W), mat(H * dv, W)
+            for nm, n in (("q", G * d), ("k", G * d), ("v", H * dv)):
+                w[x + nm + ".conv"] = (torch.randn((n, taps), device=device, generator=gen) * 0.5 + 0.25).to(dtype)
+            w[x + "b"], w[x + "A_log"], w[x + "dt_bias"] = mat(H, W), vec(H, -4.0, 0.0), vec(H * d, -4.0, -1.0)
+            w[x + "a1"], w[x + "a2"], w[x + "g1"], w[x + "g2"] = mat(decay_rank, W), mat(H * d, decay_rank), mat(gate_rank, W), mat(H * dv, gate_rank)
+            w[x + "norm"], w[x + "o"] = vec(dv, 0.9, 1.1), mat(W, H * dv)
+        else:
+            R = m["kv_rank"]
+            w[x + "q"], w[x + "uk"], w[x + "uv"], w[x + "o"] = mat(H * d, W), mat(H * d, R), mat(H * dv, R), mat(W, H * dv)
+            if "kv_from" not in m:
+                w[x + "dkv"], w[x + "dkv.norm"] = mat(R, W), vec(R, 0.9, 1.1)
+        ff, f = layer.get("mlp"), p + "mlp."
+        if ff is not None and ff["kind"] == "dense":
+            n = ff["ff"]
+            w[f + "gate"], w[f + "up"], w[f + "down"] = mat(n, W), mat(n, W), mat(W, n)
+            w[f + "gate.b"], w[f + "up.b"], w[f + "down.b"] = vec(n, -0.1, 0.1), vec(n, -0.1, 0.1), vec(W, -0.1, 0.1)
+        elif ff is not None:
+            n, E = ff["expert"]["ff"], ff["router"]["experts"]
+            w[f + "router"], w[f + "correction"] = mat(E, W, 2.0), vec(E, -0.5, 0.5)
+            for e in range(E):
+                w[f + f"e{e}.gate"], w[f + f"e{e}.up"], w[f + f"e{e}.down"] = mat(n, W), mat(n, W), mat(W, n)
+    return w
+
+
+def build_tugolix(config: Dict, device="cpu", seed: int = 0, act_dtype=torch.bfloat16, decay_rank: int = 64, gate_rank: int = 64):
+    """Random-init Tugolix with real shapes: a random checkpoint generated on ``device`` goes through the model's own ``sanitize``."""
+    from .models import tugolix
+    from .utils import load_weights
+    device = torch.device(device)
+    weights = tugolix_checkpoint(config, device, seed, decay_rank, gate_rank)
+    args = tugolix.ModelArgs.from_dict(dict(config, shapes=tugolix.Model.shapes_from(weights, config)))
+    model = tugolix.Model(args)                   # (the buffers the constructors compute -- rates, empty frequency tables -- are tiny)
+    weights = model.sanitize(weights)
+    weights = {k: (v.to(act_dtype) if v.is_floating_point() and v.dtype != torch.float32 else v) for k, v in weights.items()}
+    with torch.device("meta"):
+        model = tugolix.Model(args)
+    model = model.to_empty(device=device)
+    skipped = load_weights(model, weights, device=device)
+    if skipped:
+        raise ValueError(f"tensors without a place in the model: {skipped[:3]}")
+    model.eval()
+    return model

@@ -190,8 +190,8 @@ int gbxm_conv_tail_update(const void* y, int64_t y_stride, void* tail, const int
                           void* stream);
 /* The scan over each sequence's new rows.  r: rows of gbxm_recurrent_prepare; state fp32 [slots][H][dv][dk] (read unless the sequence
  * starts at position 0, written back); out fp32 [T][H*dv].  Per token: S <- diag(decay) S; delta: u = beta (v - S^T k) else u = v;
- * S <- S + k u^T; o = S^T q.  dk <= 256. */
-int gbxm_state_scan(const float* r, int64_t r_stride, float* state, float* out, const int32_t* seq, int32_t B, int32_t H, int32_t G,
+ * S <- S + k u^T; o = S^T q.  T: rows of the step (chooses the workgroup shape).  dk <= 256. */
+int gbxm_state_scan(const float* r, int64_t r_stride, float* state, float* out, const int32_t* seq, int32_t B, int64_t T, int32_t H, int32_t G,
                     int32_t dk, int32_t dv, int32_t delta, void* stream);
 /* out[t][h][c] = o[t][h][c] / sqrt(mean_c o^2 + eps) * w[c] * gate(g[t][h][c]); gate kind 1 silu, 2 sigmoid; o fp32, g / out activation dtype. */
 int gbxm_head_norm_gate(const float* o, const void* gate, int64_t gate_stride, const float* w, void* out, int64_t T, int32_t H, int32_t dv,
