@@ -107,7 +107,7 @@ template <int R, bool DELTA, int NW>
 __global__ __launch_bounds__(64 * NW) void state_scan_kernel(const float* __restrict__ r, int64_t r_stride, float* __restrict__ state,
                                                             float* __restrict__ out, const int* __restrict__ seq, int H, int G, int dk, int dv) {
   constexpr int DKP = 16 * R, NCOL = 4 * NW, ROW = 3 * DKP + NCOL + 1, NTH = 64 * NW;
-  constexpr int CH = (R <= 4 ? 32 : (R <= 8 ? 16 : 8)) * NW / 4;
+  constexpr int CH = NW == 1 ? (R <= 4 ? 4 : 2) : (R <= 4 ? 32 : (R <= 8 ? 16 : 8)) * NW / 4;     // one-wave workgroups serve steps of few rows
   constexpr int PF = (CH * ROW + NTH - 1) / NTH;
   __shared__ float buf[2][CH * ROW];
   const int b = blockIdx.z, h = blockIdx.y;
@@ -118,35 +118,51 @@ __global__ __launch_bounds__(64 * NW) void state_scan_kernel(const float* __rest
   const int colc = col_ok ? col : dv - 1;
   const int nq = G * dk, nv = H * dv;
   const int g = h / (H / G);
-  float* sp = state + ((static_cast<int64_t>(slot) * H + h) * dv + colc) * dk + ks;
+  float* sp = state + ((static_cast<int64_t>(slot) * H + h) * dv + colc) * dk + min(ks, dk - 1);     // (a lane past the last channel holds zeros)
+  // every load below is issued unconditionally from an address inside the buffers (what it must not deliver is replaced afterwards):
+  // loads under a branch wait for one another, and a chunk's fetch then costs the sum of their latencies
   float S[R];
 #pragma unroll
-  for (int i = 0; i < R; ++i) S[i] = (pos0 > 0 && ks + 16 * i < dk) ? sp[16 * i] : 0.f;
+  for (int i = 0; i < R; ++i) S[i] = sp[ks + 16 * i < dk ? 16 * i : 0];
+#pragma unroll
+  for (int i = 0; i < R; ++i) S[i] = (pos0 > 0 && ks + 16 * i < dk) ? S[i] : 0.f;
   const float* base = r + static_cast<int64_t>(row0) * r_stride;
   const int oq = g * dk, ok = nq + g * dk, ov = 2 * nq + h * dv, og = 2 * nq + nv + h * dk, ob = 2 * nq + nv + H * dk + h;
   float pf[PF];
-  auto fetch = [&](int t0) {
+  int offs[PF], tts[PF];                    // where slot i of this thread's share of a chunk comes from: token of the chunk, offset in its row
+  unsigned loaded = 0;                      // bit i: pf[i] is an operand (else the slot's neutral value: 1 for a decay, 0 elsewhere)
 #pragma unroll
-    for (int i = 0; i < PF; ++i) {
-      const int idx = threadIdx.x + i * NTH;
-      const int tt = idx / ROW, j = idx - tt * ROW;
-      float val = 0.f;
-      if (idx < CH * ROW && t0 + tt < n) {
-        const float* rp = base + static_cast<int64_t>(t0 + tt) * r_stride;
-        if (j < DKP) val = j < dk ? rp[oq + j] : 0.f;
-        else if (j < 2 * DKP) val = j - DKP < dk ? rp[ok + j - DKP] : 0.f;
-        else if (j < 3 * DKP) val = j - 2 * DKP < dk ? rp[og + j - 2 * DKP] : 1.f;
-        else if (j < 3 * DKP + NCOL) val = col0 + j - 3 * DKP < dv ? rp[ov + col0 + j - 3 * DKP] : 0.f;
-        else val = DELTA ? rp[ob] : 1.f;
-      }
-      pf[i] = val;
+  for (int i = 0; i < PF; ++i) {
+    const int idx = min(static_cast<int>(threadIdx.x) + i * NTH, CH * ROW - 1);
+    const int tt = idx / ROW, j = idx - tt * ROW;
+    const int seg = j < DKP ? 0 : (j < 2 * DKP ? 1 : (j < 3 * DKP ? 2 : 3));
+    const int jj = j - seg * DKP;                                     // segment 3: the value columns, then beta
+    const bool is_beta = seg == 3 && jj == NCOL;
+    const int first = seg == 0 ? oq : (seg == 1 ? ok : (seg == 2 ? og : ov + col0));
+    const int count = seg < 3 ? dk : min(dv - col0, NCOL);
+    const bool valid = is_beta ? DELTA : jj < count;
+    offs[i] = valid ? (is_beta ? ob : first + jj) : oq;
+    tts[i] = tt;
+    loaded |= static_cast<unsigned>(valid) << i;
+  }
+  auto fetch = [&](int t0) {
+    const float* cb = base + static_cast<int64_t>(t0) * r_stride;
+    if (t0 + CH <= n) {
+#pragma unroll
+      for (int i = 0; i < PF; ++i) pf[i] = cb[static_cast<int64_t>(tts[i]) * r_stride + offs[i]];
+    } else {                                // the sequence's last chunk: rows past its end are read as its last row (and never used)
+      const int last = n - 1 - t0;
+#pragma unroll
+      for (int i = 0; i < PF; ++i) pf[i] = cb[static_cast<int64_t>(min(tts[i], last)) * r_stride + offs[i]];
     }
   };
   auto park = [&](float* dst) {
 #pragma unroll
     for (int i = 0; i < PF; ++i) {
       const int idx = threadIdx.x + i * NTH;
-      if (idx < CH * ROW) dst[idx] = pf[i];
+      const int j = idx % ROW;
+      const float neutral = ((j >= 2 * DKP && j < 3 * DKP) || j == ROW - 1) ? 1.f : 0.f;
+      if (idx < CH * ROW) dst[idx] = ((loaded >> i) & 1u) ? pf[i] : neutral;
     }
   };
   fetch(0);

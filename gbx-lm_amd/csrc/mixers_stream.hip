@@ -48,7 +48,7 @@ __global__ __launch_bounds__(NT) void hyper_step_kernel(float* __restrict__ X, c
       if (!mixed) z = to_f32(yr[c]);
       else {
         z = 0.f;
-        for (int k = 0; k < top; ++k) z += (k < 64 ? ml[k] : y_mix[t * top + k]) * to_f32(yr[k * width + c]);
+        for (int k = 0; k < top; ++k) z += ml[k] * to_f32(yr[k * width + c]);
       }
 #pragma unroll
       for (int j = 0; j < MAXS; ++j) {
@@ -191,6 +191,7 @@ int gbxm_hyper_step(float* X, const void* y, const float* y_mix, const float* mi
       (norm_w ? (!norm_b || !h) : !out_u))
     return fail(GBXM_ERR_INVALID, "hyper_step: bad argument");
   if (S > MAXS) return fail(GBXM_ERR_UNSUPPORTED, "hyper_step: more than %d streams", MAXS);
+  if (top > 64) return fail(GBXM_ERR_UNSUPPORTED, "hyper_step: more than 64 candidates per row");
   const size_t lds = width > UR * NT ? static_cast<size_t>(width) * sizeof(float) : 0;
   if (lds > 60 * 1024) return fail(GBXM_ERR_UNSUPPORTED, "hyper_step: rows of %d channels", width);
   if (T_ == 0) return GBXM_OK;
