@@ -442,6 +442,32 @@ def test_unequal_batch_and_slot_reuse(checkpoints, device, dtype):
 
 
 @pytest.mark.parametrize("device", DEVICES)
+def test_slot_tables_grow_while_decoding(checkpoints, device):
+    """One sequence decodes; later three more start, one by one: the state, tail and latent tables are re-allocated with more slots
+    under the running sequence (and any captured decode step is dropped).  Every logit against the oracle."""
+    path, cfg, w = ckpt(checkpoints, "mixed", torch.float32)
+    model = model_for(checkpoints, "mixed", device, torch.float32)
+    seqs = {k: tokens_for(cfg, 26, 40 + i) for i, k in enumerate("abcd")}
+    eng = BatchScheduler(model)
+    got = {k: [] for k in seqs}
+    done = {}
+    for step in range(24):
+        if step % 6 == 0:
+            k = "abcd"[step // 6]
+            got[k].append(eng.step([(k, seqs[k][:2])], [[0, 1]]))
+            done[k] = 2
+        entries = [(k, [seqs[k][done[k]]]) for k in done if done[k] < 26]
+        out = eng.step(entries)
+        for i, (k, _) in enumerate(entries):
+            got[k].append(out[i:i + 1])
+            done[k] += 1
+    assert len(set(eng.slot_of.values())) == 4
+    for k in seqs:
+        seen = torch.cat(got[k])
+        assert O.rel_err(seen, oracle(cfg, w, seqs[k][:seen.shape[0]])[0]) < TOL[torch.float32], k
+
+
+@pytest.mark.parametrize("device", DEVICES)
 def test_long_decoding_across_table_growth(checkpoints, device):
     """300 single-token steps from the first token: the latent tables double on the way (256 rows at first), the states recur 300
     times, the decode graph is dropped and captured again when the tables move."""
