@@ -1,6 +1,6 @@
 // Recurrent mixers: a decayed matrix state per head.
 //
-//   recurrent_prep_kernel   one workgroup per row: short causal convolution + silu on q | k | v, unit q / k heads, q scale, the decay
+//   recurrent_prep_kernel   short causal convolution + silu on q | k | v, unit q / k heads (a wave per head), q scale, the decay
 //                           exp(-rate_h softplus(sign (a + bias))) and beta = sigmoid(b), all in fp32, into one fp32 row.
 //   conv_tail_kernel        the last taps-1 convolution inputs of every sequence into its slot.
 //   state_scan_kernel<R>    the scan.  The columns of a head's state (one per value channel) never meet: a wave takes four columns, 16
@@ -17,9 +17,13 @@ namespace {
 
 constexpr int NT = 256, NW = NT / 64;
 
+// grid (rows, splits): the splits of a row share out its q / k heads (a wave per head, up to MAXD channels a lane in registers),
+// its value channels, its decays and betas; a step of few rows takes more splits.  Loads are issued unconditionally (a tap before
+// the sequence's start reads a clamped address and counts as zero).
+constexpr int MAXD = 4;                     // head channels per lane: heads of up to 256 channels
+
 template <typename T, bool FAST>
 __global__ __launch_bounds__(NT) void recurrent_prep_kernel(gbxm_recurrent_prep_args p) {
-  extern __shared__ float row[];            // q | k | v of the row after convolution and silu
   const int64_t t = blockIdx.x;
   const int b = p.tok[2 * t], pos = p.tok[2 * t + 1];
   const int slot = p.seq[4 * b], pos0 = p.seq[4 * b + 1], row0 = p.seq[4 * b + 3];
@@ -27,47 +31,53 @@ __global__ __launch_bounds__(NT) void recurrent_prep_kernel(gbxm_recurrent_prep_
   const int C = 2 * nq + nv;
   const T* y = static_cast<const T*>(p.y);
   const T* yr = y + t * p.y_stride;
+  const T* cw = static_cast<const T*>(p.conv);
+  const T* tail = p.taps > 1 ? static_cast<const T*>(p.tail) + static_cast<int64_t>(slot) * (p.taps - 1) * C : nullptr;
   float* out = p.out + t * p.out_stride;
-  if (p.conv) {
-    const T* cw = static_cast<const T*>(p.conv);
-    const T* tail = static_cast<const T*>(p.tail) + static_cast<int64_t>(slot) * (p.taps - 1) * C;
-    for (int c = threadIdx.x; c < C; c += NT) {
-      float acc = 0.f;
-      for (int j = 0; j < p.taps; ++j) {
-        const int src = pos - (p.taps - 1) + j;
-        if (src < 0) continue;
-        const float x = src >= pos0 ? to_f32(y[(row0 + (src - pos0)) * p.y_stride + p.off_q + c])
-                                    : to_f32(tail[static_cast<int64_t>(src - pos0 + p.taps - 1) * C + c]);
-        acc += to_f32(cw[c * p.taps + j]) * x;
-      }
-      row[c] = acc * sigmoid_<FAST>(acc);
+  // channel c of q | k | v after the convolution and silu (or as projected, without a convolution; `plain`: its offset in the row)
+  auto value = [&](int c, int plain) {
+    if (!cw) return to_f32(yr[plain]);
+    float acc = 0.f;
+    for (int j = 0; j < p.taps; ++j) {
+      const int src = pos - (p.taps - 1) + j;
+      const bool own = src >= pos0;
+      const T* sp = own ? y + (row0 + (src - pos0)) * p.y_stride + p.off_q + c
+                        : (tail ? tail + static_cast<int64_t>(max(src, pos0 - (p.taps - 1)) - pos0 + p.taps - 1) * C + c : yr + p.off_q + c);
+      const float x = to_f32(*sp);
+      acc += src >= 0 ? to_f32(cw[c * p.taps + j]) * x : 0.f;
     }
-  } else {
-    for (int c = threadIdx.x; c < nq; c += NT) { row[c] = to_f32(yr[p.off_q + c]); row[nq + c] = to_f32(yr[p.off_k + c]); }
-    for (int c = threadIdx.x; c < nv; c += NT) row[2 * nq + c] = to_f32(yr[p.off_v + c]);
-  }
-  __syncthreads();
-  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-  // q and k heads: a wave per head
-  for (int hd = wave; hd < 2 * p.G; hd += NW) {
-    const float* v = row + hd * p.dk;
+    return acc * sigmoid_<FAST>(acc);
+  };
+  const int lane = threadIdx.x & 63;
+  const int gwave = blockIdx.y * NW + (threadIdx.x >> 6), n_waves = gridDim.y * NW;
+  const int gthread = blockIdx.y * NT + threadIdx.x, n_threads = gridDim.y * NT;
+  for (int hd = gwave; hd < 2 * p.G; hd += n_waves) {                  // q heads, then k heads
+    const int first = hd * p.dk, plain = (hd < p.G ? p.off_q + first : p.off_k + first - nq);
+    float v[MAXD];
+    float ss = 0.f;
+#pragma unroll
+    for (int i = 0; i < MAXD; ++i) {
+      const int c = lane + 64 * i;
+      const bool live = c < p.dk;
+      const float x = value(first + (live ? c : 0), plain + (live ? c : 0));
+      v[i] = live ? x : 0.f;
+      ss += v[i] * v[i];
+    }
     float mul = hd < p.G ? p.q_scale : 1.f;
-    if (p.unit) {
-      float ss = 0.f;
-      for (int c = lane; c < p.dk; c += 64) ss += v[c] * v[c];
-      mul *= 1.f / sqrtf(wave_sum(ss) + 1e-6f);
-    }
-    for (int c = lane; c < p.dk; c += 64) out[hd * p.dk + c] = v[c] * mul;
+    if (p.unit) mul *= 1.f / sqrtf(wave_sum(ss) + 1e-6f);
+#pragma unroll
+    for (int i = 0; i < MAXD; ++i)
+      if (lane + 64 * i < p.dk) out[first + lane + 64 * i] = v[i] * mul;
   }
-  for (int c = threadIdx.x; c < nv; c += NT) out[2 * nq + c] = row[2 * nq + c];
+  for (int c = gthread; c < nv; c += n_threads) out[2 * nq + c] = value(2 * nq + c, p.off_v + c);
   const T* ar = static_cast<const T*>(p.a) + t * p.a_stride;
-  for (int c = threadIdx.x; c < nd; c += NT) {
+  for (int c = gthread; c < nd; c += n_threads) {
     const float z = p.sign * (to_f32(ar[c]) + p.decay_bias[c]);
     const float sp = z > 20.f ? z : log1p_<FAST>(exp_<FAST>(z));
     out[2 * nq + nv + c] = exp_<FAST>(-p.decay_rate[c / p.dk] * sp);
   }
   if (p.off_beta >= 0)
-    for (int c = threadIdx.x; c < p.H; c += NT) out[2 * nq + nv + nd + c] = sigmoid_<FAST>(to_f32(yr[p.off_beta + c]));
+    for (int c = gthread; c < p.H; c += n_threads) out[2 * nq + nv + nd + c] = sigmoid_<FAST>(to_f32(yr[p.off_beta + c]));
 }
 
 template <typename T>
@@ -262,12 +272,18 @@ int gbxm_recurrent_prepare(const gbxm_recurrent_prep_args* a, void* stream) {
   if (a->conv && (a->taps < 1 || (a->taps > 1 && !a->tail) || a->off_k != a->off_q + nq || a->off_v != a->off_k + nq))
     return fail(GBXM_ERR_INVALID, "recurrent_prepare: a convolution needs q | k | v side by side and the slots' tails");
   if (a->out_stride < C + a->H * a->dk + (a->off_beta >= 0 ? a->H : 0)) return fail(GBXM_ERR_INVALID, "recurrent_prepare: output rows too short");
-  const size_t lds = static_cast<size_t>(C) * sizeof(float);
-  if (lds > 60 * 1024) return fail(GBXM_ERR_UNSUPPORTED, "recurrent_prepare: q | k | v rows of %d channels", C);
+  if (a->dk > 64 * MAXD) return fail(GBXM_ERR_UNSUPPORTED, "recurrent_prepare: heads of %d channels (at most %d)", a->dk, 64 * MAXD);
   if (a->T == 0) return GBXM_OK;
   hipStream_t s = static_cast<hipStream_t>(stream);
-  if (a->act == GBXM_BF16) recurrent_prep_kernel<bf16_t, false><<<dim3(a->T), NT, lds, s>>>(*a);
-  else recurrent_prep_kernel<float, false><<<dim3(a->T), NT, lds, s>>>(*a);
+  // splits of a row: enough workgroups for the chip when the step has few rows, never more than the row has work for
+  int64_t splits = (1024 + a->T - 1) / a->T;
+  const int64_t most = (C + a->H * a->dk + 4 * NT - 1) / (4 * NT);
+  if (splits > most) splits = most;
+  if (splits > 64) splits = 64;
+  if (splits < 1) splits = 1;
+  const dim3 grid(a->T, static_cast<unsigned>(splits));
+  if (a->act == GBXM_BF16) recurrent_prep_kernel<bf16_t, false><<<grid, NT, 0, s>>>(*a);
+  else recurrent_prep_kernel<float, false><<<grid, NT, 0, s>>>(*a);
   return after_launch("recurrent_prepare");
 }
 

@@ -10,20 +10,22 @@ constexpr int NT = 256, NW = NT / 64;
 constexpr int MAXS = 8;           // streams
 constexpr int UR = 8;             // read-out values a thread keeps between the passes (rows up to UR * NT wide; wider rows re-read)
 
-template <typename T>
+// S is a template parameter and every load is issued from an address inside the row (channels past the row's end are clamped, their
+// results dropped): loads under a run-time condition wait for one another, and a row would cost the sum of their latencies.
+template <typename T, int S>
 __global__ __launch_bounds__(NT) void hyper_step_kernel(float* __restrict__ X, const T* __restrict__ y, const float* __restrict__ y_mix,
                                                        const float* __restrict__ mix, const float* __restrict__ write, const float* __restrict__ read,
                                                        const float* __restrict__ norm_w, const float* __restrict__ norm_b, T* __restrict__ h,
-                                                       float* __restrict__ out_u, int S, int width, int top, float eps) {
+                                                       float* __restrict__ out_u, int width, int top, float eps) {
   __shared__ float red[NW];
-  __shared__ float sm[MAXS * MAXS + 2 * MAXS];
+  __shared__ float sm[S * S + 2 * S];
   __shared__ float ml[64];
   extern __shared__ float ul[];            // [width] when width > UR * NT, else unused
   const int64_t t = blockIdx.x;
   float* xr = X + t * S * width;
   float* mixl = sm;
-  float* wl = sm + MAXS * MAXS;
-  float* rl = wl + MAXS;
+  float* wl = sm + S * S;
+  float* rl = wl + S;
   const bool upd = y != nullptr;
   if (threadIdx.x < S * S) mixl[threadIdx.x] = upd ? mix[threadIdx.x] : 0.f;
   if (threadIdx.x < S) {
@@ -31,7 +33,7 @@ __global__ __launch_bounds__(NT) void hyper_step_kernel(float* __restrict__ X, c
     rl[threadIdx.x] = read ? read[threadIdx.x] : 1.f;
   }
   const bool mixed = y_mix != nullptr;
-  if (upd && mixed && threadIdx.x < min(top, 64)) ml[threadIdx.x] = y_mix[t * top + threadIdx.x];
+  if (upd && mixed && threadIdx.x < top) ml[threadIdx.x] = y_mix[t * top + threadIdx.x];
   __syncthreads();
   const T* yr = upd ? y + t * top * width : nullptr;
   const bool wide = width > UR * NT;
@@ -39,40 +41,38 @@ __global__ __launch_bounds__(NT) void hyper_step_kernel(float* __restrict__ X, c
   float sum = 0.f;
   // pass 1: the update of every channel's S values (a channel is independent of the others) and the read-out u
   auto channel = [&](int c) {
-    float xs[MAXS];
+    const bool live = c < width;
+    const int cc = live ? c : width - 1;
+    float xs[S];
 #pragma unroll
-    for (int i = 0; i < MAXS; ++i) xs[i] = i < S ? xr[i * width + c] : 0.f;
+    for (int i = 0; i < S; ++i) xs[i] = xr[i * width + cc];
     float u = 0.f;
     if (upd) {
       float z;
-      if (!mixed) z = to_f32(yr[c]);
+      if (!mixed) z = to_f32(yr[cc]);
       else {
         z = 0.f;
-        for (int k = 0; k < top; ++k) z += ml[k] * to_f32(yr[k * width + c]);
+        for (int k = 0; k < top; ++k) z += ml[k] * to_f32(yr[k * width + cc]);
       }
 #pragma unroll
-      for (int j = 0; j < MAXS; ++j) {
-        if (j < S) {
-          float v = 0.f;
+      for (int j = 0; j < S; ++j) {
+        float v = 0.f;
 #pragma unroll
-          for (int i = 0; i < MAXS; ++i)
-            if (i < S) v += mixl[i * S + j] * xs[i];
-          v += wl[j] * z;
-          xr[j * width + c] = v;
-          u += rl[j] * v;
-        }
+        for (int i = 0; i < S; ++i) v += mixl[i * S + j] * xs[i];
+        v += wl[j] * z;
+        if (live) xr[j * width + cc] = v;
+        u += rl[j] * v;
       }
     } else {
 #pragma unroll
-      for (int j = 0; j < MAXS; ++j)
-        if (j < S) u += rl[j] * xs[j];
+      for (int j = 0; j < S; ++j) u += rl[j] * xs[j];
     }
-    return u;
+    return live ? u : 0.f;
   };
 #pragma unroll
   for (int i = 0; i < UR; ++i) {
     const int c = threadIdx.x + i * NT;
-    ur[i] = c < width ? channel(c) : 0.f;
+    ur[i] = channel(c);
     sum += ur[i];
     if (wide && c < width) ul[c] = ur[i];
   }
@@ -101,6 +101,24 @@ __global__ __launch_bounds__(NT) void hyper_step_kernel(float* __restrict__ X, c
     if (c < width) h[t * width + c] = from_f32<T>((ur[i] - mean) * r * norm_w[c] + norm_b[c]);
   }
   for (int c = threadIdx.x + UR * NT; c < width; c += NT) h[t * width + c] = from_f32<T>((ul[c] - mean) * r * norm_w[c] + norm_b[c]);
+}
+
+template <typename T>
+void launch_hyper_step(int S, dim3 grid, size_t lds, hipStream_t s, float* X, const void* y, const float* y_mix, const float* mix, const float* write,
+                       const float* read, const float* norm_w, const float* norm_b, void* h, float* out_u, int width, int top, float eps) {
+#define GBXM_HS(N) hyper_step_kernel<T, N><<<grid, NT, lds, s>>>(X, static_cast<const T*>(y), y_mix, mix, write, read, norm_w, norm_b, static_cast<T*>(h), \
+                                                               out_u, width, top, eps)
+  switch (S) {
+    case 1: GBXM_HS(1); break;
+    case 2: GBXM_HS(2); break;
+    case 3: GBXM_HS(3); break;
+    case 4: GBXM_HS(4); break;
+    case 5: GBXM_HS(5); break;
+    case 6: GBXM_HS(6); break;
+    case 7: GBXM_HS(7); break;
+    default: GBXM_HS(8); break;
+  }
+#undef GBXM_HS
 }
 
 template <typename T, bool FAST>
@@ -196,12 +214,8 @@ int gbxm_hyper_step(float* X, const void* y, const float* y_mix, const float* mi
   if (lds > 60 * 1024) return fail(GBXM_ERR_UNSUPPORTED, "hyper_step: rows of %d channels", width);
   if (T_ == 0) return GBXM_OK;
   hipStream_t s = static_cast<hipStream_t>(stream);
-  if (act == GBXM_BF16)
-    hyper_step_kernel<bf16_t><<<dim3(T_), NT, lds, s>>>(X, static_cast<const bf16_t*>(y), y_mix, mix, write, read, norm_w, norm_b,
-                                                       static_cast<bf16_t*>(h), out_u, S, width, top, eps);
-  else
-    hyper_step_kernel<float><<<dim3(T_), NT, lds, s>>>(X, static_cast<const float*>(y), y_mix, mix, write, read, norm_w, norm_b,
-                                                      static_cast<float*>(h), out_u, S, width, top, eps);
+  if (act == GBXM_BF16) launch_hyper_step<bf16_t>(S, dim3(T_), lds, s, X, y, y_mix, mix, write, read, norm_w, norm_b, h, out_u, width, top, eps);
+  else launch_hyper_step<float>(S, dim3(T_), lds, s, X, y, y_mix, mix, write, read, norm_w, norm_b, h, out_u, width, top, eps);
   return after_launch("hyper_step");
 }
 
