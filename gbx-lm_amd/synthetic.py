@@ -373,7 +373,7 @@ def tugolix_config(width: int, delta: Dict, gla: Dict, latent: Dict, ff: int, mo
     feed-forward of ``ff`` channels, the others the routed one.  ``delta``: heads, kv_heads, dim, vdim, conv; ``gla``: heads, dim, vdim,
     tau; ``latent``: heads, dim, vdim, kv_rank; ``moe``: experts, top, ff, groups (count, keep), limit, scale."""
     routed = {"kind": "moe", "expert": {"ff": moe["ff"], "limit": moe.get("limit", 7.0)},
-              "router": {"experts": moe["experts"], "top": moe["top"], "scale": moe.get("scale", 2.5),
+              "router": {"experts": moe["experts"], "top": moe["top"], "scale": moe.get("scale", 1.0),
                          "groups": {"count": moe["groups"][0], "keep": moe["groups"][1]}}}
     layers, owner = [], None
     for i, c in enumerate(pattern):
