@@ -184,7 +184,8 @@ class BatchScheduler:
         for c in self.caches:                            # tables without a window grow on the host, never inside a replay
             if hasattr(c, "ensure"):
                 c.ensure(longest)
-        buffers = tuple(c.keys.data_ptr() if c.keys is not None else 0 for c in self.caches)
+        buffers = tuple(b.data_ptr() if b is not None else 0 for c in self.caches
+                        for b in (c.buffers() if hasattr(c, "buffers") else (c.keys,)))
         if buffers != self._buffers:                     # rings were (re)allocated: every captured pointer is stale
             self._graphs.clear()
             self._seen.clear()

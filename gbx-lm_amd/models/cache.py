@@ -318,3 +318,87 @@ class SlotStateCache:
 
     def is_trimmable(self):
         return False
+
+
+class SlotRowCache:
+    """One row of ``width`` values per slot: what a sequence's last token leaves for its next one (the previous token's id for a
+    hashed pair embedding, the previous token's normed input for a token shift).  ``kind`` is "act" (the activation dtype of the
+    first reserve), "f32" or "i64".  As with the other slot tables a slot is not cleared when it is handed out again: a sequence
+    at position 0 has no previous token by position, never by the buffer's contents."""
+
+    def __init__(self, width: int, kind: str = "act", slots: Optional[SequenceSlots] = None):
+        if kind not in ("act", "f32", "i64"):
+            raise ValueError("SlotRowCache: kind is act, f32 or i64")
+        self.width, self.kind = int(width), kind
+        self.slots = slots if slots is not None else SequenceSlots(1)
+        self.slots.listeners.append(self)
+        self.rows = None
+
+    @property
+    def keys(self):
+        return self.rows
+
+    @property
+    def offset(self) -> int:
+        return max(self.slots.length[0], 0)
+
+    def reserve(self, dtype, device) -> None:
+        if self.rows is None:
+            dt = {"act": dtype, "f32": torch.float32, "i64": torch.int64}[self.kind]
+            self.rows = torch.zeros((self.slots.n_slots, self.width), dtype=dt, device=device)
+
+    def grow(self, n_slots: int) -> None:
+        if self.rows is not None and self.rows.shape[0] < n_slots:
+            new = torch.zeros((max(n_slots, 2 * self.rows.shape[0]), self.width), dtype=self.rows.dtype, device=self.rows.device)
+            new[:self.rows.shape[0]] = self.rows
+            self.rows = new
+
+    def is_trimmable(self):
+        return False
+
+
+class CacheGroup:
+    """The cache entry of a layer that carries more than one kind of state (say a token shift's row next to its mixer's table, or
+    the two tables of two mixers side by side): named parts over ONE slot table.  ``buffers`` lists every device buffer a captured
+    step depends on; ``ensure`` reaches the parts that can grow in rows."""
+
+    def __init__(self, slots: SequenceSlots, **parts):
+        self.slots = slots
+        self.parts = dict(parts)
+        for name, part in parts.items():
+            if part is not None and part.slots is not slots:
+                raise ValueError("CacheGroup: every part lives on the group's slot table")
+            setattr(self, name, part)
+
+    def _leaves(self):
+        for part in self.parts.values():
+            if isinstance(part, CacheGroup):
+                yield from part._leaves()
+            elif part is not None:
+                yield part
+
+    def buffers(self):
+        out = []
+        for c in self._leaves():
+            for nm in ("keys", "values", "tail"):
+                t = getattr(c, nm, None)
+                if nm == "keys" or (t is not None and t.numel()):
+                    out.append(t)
+        return out
+
+    @property
+    def keys(self):                              # None until every part has its buffers
+        bufs = self.buffers()
+        return None if any(b is None for b in bufs) or not bufs else bufs[0]
+
+    @property
+    def offset(self) -> int:
+        return max(self.slots.length[0], 0)
+
+    def ensure(self, longest: int) -> None:
+        for c in self._leaves():
+            if hasattr(c, "ensure"):
+                c.ensure(longest)
+
+    def is_trimmable(self):
+        return False

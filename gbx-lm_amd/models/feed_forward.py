@@ -44,12 +44,32 @@ class DenseFeedForward(nn.Module):
         return F.linear(activate_(F.linear(h, self.up.weight), self.activation), self.down.weight)
 
 
-GLU_KINDS = ("silu", "clamped_swish")
+GLU_KINDS = ("silu", "clamped_swish", "gelu_tanh", "sigmoid")
+
+
+def _gate_act(g: torch.Tensor, kind: str) -> torch.Tensor:
+    if kind == "silu":
+        return F.silu(g)
+    if kind == "sigmoid":
+        return torch.sigmoid(g)
+    return 0.5 * g * (1.0 + torch.tanh(math.sqrt(2.0 / math.pi) * (g + 0.044715 * g.pow(3))))
+
+
+def gate_mul(gate: torch.Tensor, up: torch.Tensor, kind: str) -> torch.Tensor:
+    """act(gate) * up over rows [T, F] that need not be neighbours in memory (unit inner stride), fp32 arithmetic, a new tensor in
+    the rows' dtype.  ``kind``: silu, sigmoid or gelu_tanh."""
+    if kind not in ("silu", "sigmoid", "gelu_tanh"):
+        raise ValueError(f"unknown gate activation {kind!r}")
+    if gate.is_cuda:
+        from .. import mixer_ops as M
+        return M.gate_mul(gate, up, kind)
+    return (_gate_act(gate.float(), kind) * up.float()).to(up.dtype)
 
 
 def glu_(gu: torch.Tensor, kind: str = "silu", limit: float = 0.0, alpha: float = 1.702) -> torch.Tensor:
     """Rows ``gu`` [T, 2F] = gate | up  ->  [T, F] in the same dtype, fp32 arithmetic.  ``silu``: g sigmoid(g) u.  ``clamped_swish``:
-    g' = min(g, limit), u' = clamp(u, -limit, limit), g' sigmoid(alpha g') (u' + 1)."""
+    g' = min(g, limit), u' = clamp(u, -limit, limit), g' sigmoid(alpha g') (u' + 1).  ``gelu_tanh``: gelu(g) u in the tanh form.
+    ``sigmoid``: sigmoid(g) u."""
     if kind not in GLU_KINDS:
         raise ValueError(f"unknown gated activation {kind!r}")
     if gu.is_cuda:
@@ -57,14 +77,15 @@ def glu_(gu: torch.Tensor, kind: str = "silu", limit: float = 0.0, alpha: float 
         return M.glu(gu, kind, limit, alpha)
     f = gu.shape[-1] // 2
     g, u = gu[..., :f].float(), gu[..., f:].float()
-    if kind == "silu":
-        return (F.silu(g) * u).to(gu.dtype)
+    if kind != "clamped_swish":
+        return (_gate_act(g, kind) * u).to(gu.dtype)
     g, u = g.clamp(max=limit), u.clamp(min=-limit, max=limit)
     return (g * torch.sigmoid(alpha * g) * (u + 1.0)).to(gu.dtype)
 
 
 class GatedDenseFeedForward(nn.Module):
-    """``down(silu(gate h + b_g) * (up h + b_u)) + b_d``; gate and up are one product (rows gate | up)."""
+    """``down(act(gate h + b_g) * (up h + b_u)) + b_d``; gate and up are one product (rows gate | up); ``kind`` names the gate's
+    activation (silu, gelu_tanh); ``bias=False``: no biases."""
 
     def __init__(self, width: int, ff: int, bias: bool = True, kind: str = "silu"):
         super().__init__()

@@ -15,7 +15,8 @@ scaled to unit length per head, q times a constant, the decay  g = exp(-rate_h *
 exp(A_h)`` -- and ``beta = sigmoid(b)``.  After the scan each head's read-out is RMS-normalised over its value channels, weighted
 and gated (``head_norm_gate``: silu or sigmoid gate).
 
-Mixers: ``GatedLinearAttention`` (plain write, decay from a low-rank projection, silu output gate) and ``ChannelDeltaRule`` (delta
+Mixers: ``GatedLinearAttention`` (plain write, decay from a low-rank projection, silu output gate), ``LightningAttention`` (plain
+write, silu on q / k / v, a constant decay per head, all heads normalised together, sigmoid gate) and ``ChannelDeltaRule`` (delta
 write with grouped q / k heads, convolution, unit q / k, low-rank decay and low-rank sigmoid gate).
 
 GPU tensors run the HIP kernels of ``mixer_ops``; CPU tensors the plain torch graph below, which the kernels are tested against.
@@ -56,16 +57,21 @@ class RecurrentLayout:
     def out_width(self) -> int: return 2 * self.nq + self.nv + self.nd + (self.heads if self.off_beta >= 0 else 0)
 
 
-def recurrent_prepare(y: torch.Tensor, a: torch.Tensor, lay: RecurrentLayout, decay_bias: torch.Tensor, decay_rate: torch.Tensor, sign: float,
-                      conv: Optional[torch.Tensor], cache: SlotStateCache, batch, unit: bool, q_scale: float) -> torch.Tensor:
+def recurrent_prepare(y: torch.Tensor, a: Optional[torch.Tensor], lay: RecurrentLayout, decay_bias: Optional[torch.Tensor], decay_rate: torch.Tensor,
+                      sign: float, conv: Optional[torch.Tensor], cache: SlotStateCache, batch, unit: bool, q_scale: float,
+                      qkv_silu: bool = False) -> torch.Tensor:
     """y [T, N] projection rows, a [T, heads * dk] decay projection rows (both activation dtype, unit inner stride) -> fp32
-    [T, q | k | v | decay | beta].  ``conv`` [nq + nq + nv, taps] or None (then q | k | v must be adjacent from ``off_q`` on)."""
+    [T, q | k | v | decay | beta].  ``conv`` [nq + nq + nv, taps] or None (then q | k | v must be adjacent from ``off_q`` on).
+    ``a`` None: no decay projection, every key channel of head h decays by the constant ``decay_rate[h]`` itself.  ``qkv_silu``
+    (without a convolution): q, k and v pass silu."""
     if y.is_cuda:
         from .. import mixer_ops as M
-        return M.recurrent_prepare(y, a, lay, decay_bias, decay_rate, sign, conv, cache, batch, unit, q_scale)
+        return M.recurrent_prepare(y, a, lay, decay_bias, decay_rate, sign, conv, cache, batch, unit, q_scale, qkv_silu)
     t = y.shape[0]
     nq, nv = lay.nq, lay.nv
     q, k, v = y[:, lay.off_q:lay.off_q + nq].float(), y[:, lay.off_k:lay.off_k + nq].float(), y[:, lay.off_v:lay.off_v + nv].float()
+    if qkv_silu and conv is None:
+        q, k, v = F.silu(q), F.silu(k), F.silu(v)
     if conv is not None:
         taps = conv.shape[1]
         raw = torch.cat([q, k, v], dim=1)
@@ -88,8 +94,11 @@ def recurrent_prepare(y: torch.Tensor, a: torch.Tensor, lay: RecurrentLayout, de
         k = k.view(t, lay.groups, lay.dk)
         q = (q * torch.rsqrt(q.pow(2).sum(-1, keepdim=True) + 1e-6)).reshape(t, nq)
         k = (k * torch.rsqrt(k.pow(2).sum(-1, keepdim=True) + 1e-6)).reshape(t, nq)
-    z = sign * (a.float() + decay_bias.float())
-    decay = torch.exp(-decay_rate.float().repeat_interleave(lay.dk)[None, :] * F.softplus(z))
+    if a is None:
+        decay = decay_rate.float().repeat_interleave(lay.dk)[None, :].expand(t, lay.nd)
+    else:
+        z = sign * (a.float() + decay_bias.float())
+        decay = torch.exp(-decay_rate.float().repeat_interleave(lay.dk)[None, :] * F.softplus(z))
     parts = [q * q_scale, k, v, decay]
     if lay.off_beta >= 0:
         parts.append(torch.sigmoid(y[:, lay.off_beta:lay.off_beta + lay.heads].float()))
@@ -159,10 +168,12 @@ def _pad8(n: int) -> int:
 
 
 class _RecurrentMixer(nn.Module):
-    """Shared by the two mixers: the cache and the order of launches of a step."""
+    """Shared by the mixers: the cache and the order of launches of a step."""
     delta = False
     unit = False
     gate_kind = GATE_SILU
+    qkv_silu = False
+    norm_heads_together = False        # the read-outs of all heads are RMS-normalised as ONE vector (weight over heads * dv)
 
     def make_cache(self, slots) -> SlotStateCache:
         lay = self.layout
@@ -172,11 +183,11 @@ class _RecurrentMixer(nn.Module):
         lay = self.layout
         cache.reserve(y.dtype, y.device)
         r = recurrent_prepare(y, a, lay, self.decay_bias, self.decay_rate, self.decay_sign, self.conv if self.taps else None, cache, batch,
-                              self.unit, self.q_scale)
+                              self.unit, self.q_scale, self.qkv_silu)
         if self.taps > 1:
             conv_tail_update(y, 2 * lay.nq + lay.nv, cache, batch)
         o = decayed_state_scan(r, lay, cache, batch, self.delta)
-        return F.linear(head_norm_gate(o, gate, self.out_norm, lay.heads, self.eps, self.gate_kind), self.o.weight)
+        return F.linear(head_norm_gate(o, gate, self.out_norm, 1 if self.norm_heads_together else lay.heads, self.eps, self.gate_kind), self.o.weight)
 
 
 class GatedLinearAttention(_RecurrentMixer):
@@ -203,6 +214,36 @@ class GatedLinearAttention(_RecurrentMixer):
         y = F.linear(h, self.inp.weight)
         a = F.linear(y[:, self.off_a1:self.off_a1 + self.decay_rank], self.a2.weight)
         return self._mix(y, a, y[:, self.off_gate:self.off_gate + self.layout.nv], batch, cache)
+
+
+class LightningAttention(_RecurrentMixer):
+    """q = silu(W_q h), k = silu(W_k h), v = silu(W_v h) per head; every key channel of head h decays by the constant ``decay[h]``;
+    plain write, no scale; the read-outs of all heads are RMS-normalised together (one weight over heads * vdim), times
+    sigmoid(W_g h); then W_o."""
+    gate_kind = GATE_SIGMOID
+    qkv_silu = True
+    norm_heads_together = True
+
+    def __init__(self, width: int, heads: int, dim: int, vdim: int, decay, eps: float):
+        super().__init__()
+        if len(decay) != heads:
+            raise ValueError("LightningAttention: one decay per head")
+        self.width, self.eps, self.taps = width, float(eps), 0
+        nq, nv = heads * dim, heads * vdim
+        self.layout = RecurrentLayout(heads, heads, dim, vdim, 0, nq, 2 * nq)
+        self.off_gate = 2 * nq + nv
+        self.inp = nn.Linear(width, _pad8(self.off_gate + nv), bias=False)                # q | k | v | g
+        self.o = nn.Linear(nv, width, bias=False)
+        self.decay_bias = None
+        self.register_buffer("decay_rate", torch.tensor([float(d) for d in decay], dtype=torch.float64).to(torch.float32))
+        self.register_buffer("out_norm", torch.ones(nv))
+        self.decay_sign, self.q_scale = 0.0, 1.0
+        for p in self.parameters():
+            p.requires_grad_(False)
+
+    def forward(self, h: torch.Tensor, batch, cache: SlotStateCache) -> torch.Tensor:
+        y = F.linear(h, self.inp.weight)
+        return self._mix(y, None, y[:, self.off_gate:self.off_gate + self.layout.nv], batch, cache)
 
 
 class ChannelDeltaRule(_RecurrentMixer):

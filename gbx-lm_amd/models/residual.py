@@ -3,6 +3,9 @@
 Branch-norm form:  x <- x + mult * rms_norm(branch) * weight.  Parallel form: ``stream_add_`` / ``stream_add_norm_``.  Several
 streams (``hyper_step_``): a sublayer reads a weighted sum of ``s`` streams and its output is written to all of them while a small
 matrix mixes the streams among themselves.  ``StreamRMSNorm`` / ``StreamLayerNorm`` turn stream rows into sublayer inputs.
+Sandwich form (a norm in front of AND behind every sublayer): ``branch_norm_add_norm_`` is the update by a normed branch together
+with the next sublayer's norm, ``norm_token_shift`` the norm in front of a mixer that also reads the previous token's norm,
+``normed_pair_mean`` the mean of two separately normed branches.
 
 The stream ``x`` is fp32 whatever the activation dtype is (it is a long sum of small terms); the branch arrives in the activation
 dtype, either as rows [T, W] or as ``top`` candidate rows per token [T, top, W] with fp32 mixing weights [T, top] (the routed
@@ -104,3 +107,56 @@ def hyper_step_(streams: torch.Tensor, y: Optional[torch.Tensor], y_mix: Optiona
     mean = u.mean(-1, keepdim=True)
     var = (u - mean).pow(2).mean(-1, keepdim=True)
     return ((u - mean) * torch.rsqrt(var + norm.eps) * norm.weight.float() + norm.bias.float()).to(act_dtype)
+
+
+def norm_token_shift(x: torch.Tensor, weight: torch.Tensor, eps: float, shift: torch.Tensor, cache, batch, act_dtype: torch.dtype) -> torch.Tensor:
+    """RMS norm of fp32 stream rows followed by a token shift, as one launch on the GPU:
+
+        n_t = x_t / sqrt(mean(x_t^2) + eps) * weight,      h_t = n_t + (n_(t-1) - n_t) * shift     (n_(-1) = 0)
+
+    ``n_(t-1)`` of a step's first row comes from ``cache`` (a ``SlotRowCache`` of fp32 rows: the norm of the sequence's last token,
+    which this call leaves there for the next step).  Everything in fp32; returns h in ``act_dtype``."""
+    cache.reserve(act_dtype, x.device)
+    if x.is_cuda:
+        from .. import mixer_ops as M
+        return M.norm_token_shift(x, weight, eps, shift, cache.rows, batch, act_dtype)
+    n = x * torch.rsqrt(x.pow(2).mean(-1, keepdim=True) + eps) * weight.float()
+    prev = torch.empty_like(n)
+    r0 = 0
+    for slot, pos0, cnt in zip(batch.slot, batch.pos0, batch.n_new):
+        prev[r0] = cache.rows[slot] if pos0 else 0.0
+        prev[r0 + 1:r0 + cnt] = n[r0:r0 + cnt - 1]
+        cache.rows[slot] = n[r0 + cnt - 1]
+        r0 += cnt
+    return (n + (prev - n) * shift.float()).to(act_dtype)
+
+
+def branch_norm_add_norm_(x: torch.Tensor, branch: torch.Tensor, mix: Optional[torch.Tensor], extra: Optional[torch.Tensor], weight: torch.Tensor,
+                          eps: float, next_weight: Optional[torch.Tensor], act_dtype: torch.dtype) -> Optional[torch.Tensor]:
+    """x += rms_norm(z) * weight in place on the fp32 stream, z = branch [T, W] -- or sum_k mix[t, k] branch[t, k] for candidate rows
+    [T, top, W] with fp32 weights [T, top] -- plus ``extra`` [T, W] if given (a branch every token takes, e.g. a shared expert); then,
+    with ``next_weight``, returns rms_norm(x) * next_weight in ``act_dtype`` (the next sublayer's input): one launch on the GPU."""
+    if x.is_cuda:
+        from .. import mixer_ops as M
+        return M.branch_norm_add_norm_(x, branch, mix, extra, weight, eps, next_weight, act_dtype)
+    z = branch.float()
+    if mix is not None:
+        z = (z * mix.float().unsqueeze(-1)).sum(1)
+    if extra is not None:
+        z = z + extra.float()
+    x.add_(z * torch.rsqrt(z.pow(2).mean(-1, keepdim=True) + eps) * weight.float())
+    if next_weight is None:
+        return None
+    return (x * torch.rsqrt(x.pow(2).mean(-1, keepdim=True) + eps) * next_weight.float()).to(act_dtype)
+
+
+def normed_pair_mean(a: torch.Tensor, b: torch.Tensor, wa: torch.Tensor, wb: torch.Tensor, eps: float) -> torch.Tensor:
+    """(rms_norm(a) * wa + rms_norm(b) * wb) / 2 over rows [T, W] in fp32, result in the rows' dtype: the output of two mixers that
+    run side by side."""
+    if a.is_cuda:
+        from .. import mixer_ops as M
+        return M.normed_pair_mean(a, b, wa, wb, eps)
+    fa, fb = a.float(), b.float()
+    na = fa * torch.rsqrt(fa.pow(2).mean(-1, keepdim=True) + eps) * wa.float()
+    nb = fb * torch.rsqrt(fb.pow(2).mean(-1, keepdim=True) + eps) * wb.float()
+    return (0.5 * (na + nb)).to(a.dtype)

@@ -9,6 +9,8 @@ Scores, weights and the running sums are 32-bit whatever the activation dtype is
 
 Mixers:
 
+* ``GatedSinkWindowAttention``: grouped-query attention with biases; weighted q / k norm per head before a partial rotation, unit
+  values, sliding window, learned sink per head, a sigmoid output gate per channel.
 * ``RotatedValueWindowAttention``: grouped-query attention; q and k are rotated (rotate-half pairs over the first ``rot_dims``
   channels, any frequency table) and then set to unit root mean square per head; values are rotated by their own position over all
   of their channels and cached so, a head's output is turned back by the query's position (so a value enters rotated by the
@@ -41,7 +43,8 @@ class HeadSegment:
     """A run of ``heads`` heads of ``head_dim`` channels inside a row, starting at ``offset``: what ``rotate_norm_heads_`` does to it.
     Channels [rot_offset, rot_offset + rot_dims) of every head are rotated (pair i with i + rot_dims / 2, or 2i with 2i + 1 when
     ``interleaved``) by ``sign * position * freq[i]``, cos and sin times ``mult``; then the head is normalised to unit root mean
-    square (NORM_UNIT) or RMS-normalised with a weight per channel (NORM_WEIGHT)."""
+    square (NORM_UNIT) or RMS-normalised with a weight per channel (NORM_WEIGHT).  ``norm_first``: the norm comes before the
+    rotation (the weight then meets the channels as projected)."""
     offset: int
     heads: int
     head_dim: int
@@ -53,6 +56,7 @@ class HeadSegment:
     interleaved: bool = False
     norm: int = NORM_NONE
     weight: Optional[torch.Tensor] = None
+    norm_first: bool = False
 
 
 def rotate_norm_heads_(rows: torch.Tensor, positions: torch.Tensor, segments: List[HeadSegment], eps: float) -> None:
@@ -66,6 +70,12 @@ def rotate_norm_heads_(rows: torch.Tensor, positions: torch.Tensor, segments: Li
     for s in segments:
         seg = rows[:, s.offset:s.offset + s.heads * s.head_dim].view(t, s.heads, s.head_dim)
         v = seg.float()
+
+        def normed(v):
+            v = v * torch.rsqrt(v.pow(2).mean(-1, keepdim=True) + eps)
+            return v * s.weight.float() if s.norm == NORM_WEIGHT else v
+        if s.norm != NORM_NONE and s.norm_first:
+            v = normed(v)
         if s.rot_dims:
             a = s.sign * (pos[:, None] * s.freq.float()[None, :])
             cos, sin = (torch.cos(a) * s.mult)[:, None, :], (torch.sin(a) * s.mult)[:, None, :]
@@ -77,10 +87,8 @@ def rotate_norm_heads_(rows: torch.Tensor, positions: torch.Tensor, segments: Li
                 u, w = part[..., :s.rot_dims // 2], part[..., s.rot_dims // 2:]
                 turned = torch.cat([u * cos - w * sin, w * cos + u * sin], dim=-1)
             v = torch.cat([v[..., :s.rot_offset], turned, v[..., s.rot_offset + s.rot_dims:]], dim=-1)
-        if s.norm != NORM_NONE:
-            v = v * torch.rsqrt(v.pow(2).mean(-1, keepdim=True) + eps)
-            if s.norm == NORM_WEIGHT:
-                v = v * s.weight.float()
+        if s.norm != NORM_NONE and not s.norm_first:
+            v = normed(v)
         seg.copy_(v.to(rows.dtype))
 
 
@@ -197,6 +205,63 @@ class RotatedValueWindowAttention(nn.Module):
         rotate_norm_heads_(ctx, pos, [HeadSegment(0, self.heads, self.vdim, 0, self.vdim, self.vfreq, sign=-1.0)], self.eps)
         cache_append(cache, k_rows, v_rows, batch)
         return F.linear(ctx, self.o.weight)
+
+
+class GatedSinkWindowAttention(nn.Module):
+    """Grouped-query sliding-window attention: q | k | v (and the gate) from one projection with biases; q and k RMS-normalised per
+    head with a weight per channel BEFORE the rotation; rotate-half pairs over the first ``rot_dims`` channels of a head (any
+    frequency table: plain, linear, YaRN); every value head scaled to unit root mean square and cached so; scores times ``scale``;
+    window ``i - j < window`` (None: all earlier keys); a learned sink per head in the softmax denominator; the concatenated heads
+    times sigmoid(W_g h), channel by channel; output projection with a bias."""
+
+    def __init__(self, width: int, heads: int, kv_heads: int, dim: int, vdim: int, rot_dims: int, rot_base: float,
+                 rot_scaling: Optional[dict], window: Optional[int], scale: float, eps: float, bias: bool = True):
+        super().__init__()
+        if heads % kv_heads or rot_dims % 2 or rot_dims > dim:
+            raise ValueError("heads must be a multiple of kv_heads; the rotated channel count is even and within the head")
+        self.width, self.heads, self.kv_heads, self.dim, self.vdim = width, heads, kv_heads, dim, vdim
+        self.window = None if window is None else int(window)
+        self.scale, self.eps, self.rot_dims = float(scale), float(eps), int(rot_dims)
+        self.nq, self.nk, self.nv, self.ng = heads * dim, kv_heads * dim, kv_heads * vdim, heads * vdim
+        self.off_gate = (self.nq + self.nk + self.nv + 7) // 8 * 8
+        self.inp = nn.Linear(width, (self.off_gate + self.ng + 7) // 8 * 8, bias=bias)          # q | k | v | (empty rows) | g
+        self.o = nn.Linear(self.ng, width, bias=bias)
+        freq, self.rot_mult = rotary_table(rot_base, rot_dims, rot_scaling) if rot_dims else (torch.zeros(0), 1.0)
+        self.register_buffer("freq", freq)
+        self.register_buffer("q_norm", torch.ones(dim))
+        self.register_buffer("k_norm", torch.ones(dim))
+        self.register_buffer("sink", torch.zeros(heads))
+        for p in self.parameters():
+            p.requires_grad_(False)
+
+    def make_cache(self, slots) -> SlotKVCache:
+        return SlotKVCache(self.nk, self.nv, self.window, 0, slots)
+
+    def fuse_weights(self, q, k, v, g, qb=None, kb=None, vb=None):
+        """The input projection (and its bias) from the checkpoint's matrices (all [out, in]), with the empty rows in front of the gate."""
+        w = torch.zeros((self.inp.out_features, q.shape[1]), dtype=q.dtype, device=q.device)
+        b = torch.zeros((self.inp.out_features,), dtype=q.dtype, device=q.device)
+        for off, part, bias in ((0, q, qb), (self.nq, k, kb), (self.nq + self.nk, v, vb), (self.off_gate, g, None)):
+            w[off:off + part.shape[0]] = part
+            if bias is not None:
+                b[off:off + part.shape[0]] = bias
+        return w, b
+
+    def forward(self, h: torch.Tensor, batch, cache: SlotKVCache) -> torch.Tensor:
+        from .feed_forward import gate_mul
+        t = h.shape[0]
+        y = F.linear(h, self.inp.weight, self.inp.bias)
+        pos = batch.tok[:, 1]
+        rotate_norm_heads_(y, pos, [
+            HeadSegment(0, self.heads, self.dim, 0, self.rot_dims, self.freq, self.rot_mult, norm=NORM_WEIGHT, weight=self.q_norm, norm_first=True),
+            HeadSegment(self.nq, self.kv_heads, self.dim, 0, self.rot_dims, self.freq, self.rot_mult, norm=NORM_WEIGHT, weight=self.k_norm, norm_first=True),
+            HeadSegment(self.nq + self.nk, self.kv_heads, self.vdim, norm=NORM_UNIT)], self.eps)
+        cache.reserve(max(p + n for p, n in zip(batch.pos0, batch.n_new)), y.dtype, y.device)
+        k_rows, v_rows = y[:, self.nq:self.nq + self.nk], y[:, self.nq + self.nk:self.nq + self.nk + self.nv]
+        ctx = sink_attend(y[:, :self.nq].view(t, self.heads, self.dim), k_rows.view(t, self.kv_heads, self.dim),
+                          v_rows.view(t, self.kv_heads, self.vdim), cache, batch, self.scale, self.window, 0, self.sink)
+        cache_append(cache, k_rows, v_rows, batch)
+        return F.linear(gate_mul(y[:, self.off_gate:self.off_gate + self.ng], ctx, "sigmoid"), self.o.weight, self.o.bias)
 
 
 class LatentAttention(nn.Module):

@@ -18,12 +18,13 @@ from typing import Any, Callable, Generator, List, Optional, Tuple, Type, Union
 import torch
 from torch import nn
 
-from .models import qdeepseek_v3, qllama, qmixtral, qphi3, qqwen2, qqwen3, qqwen3_moe, radenex, revitar, tugolix
+from .models import laruzen, qdeepseek_v3, qllama, qmixtral, qphi3, qqwen2, qqwen3, qqwen3_moe, radenex, revitar, tugolix
 from .models import cache as cache_mod
 from .models.quantized_linear_gba import QuantizedLinear
 from .tokenizer_utils import TokenizerWrapper, load_tokenizer
 
 MODEL_MAPPING = {
+    "laruzen": laruzen,       # dense checkpoint in sandwich-norm form: recurrent, linear-attention and parallel mixers, named by "architecture"
     "llama": qllama,
     "mistral": qllama,  # utils.py:52-61 maps mistral onto the llama graph
     "deepseek_v3": qdeepseek_v3,
