@@ -339,7 +339,7 @@ class RecurrentPrepArgs(ctypes.Structure):
                 ("T", ctypes.c_int64), ("H", ctypes.c_int32), ("G", ctypes.c_int32), ("dk", ctypes.c_int32), ("dv", ctypes.c_int32),
                 ("off_q", ctypes.c_int32), ("off_k", ctypes.c_int32), ("off_v", ctypes.c_int32), ("off_beta", ctypes.c_int32),
                 ("taps", ctypes.c_int32), ("unit", ctypes.c_int32), ("sign", ctypes.c_float), ("q_scale", ctypes.c_float),
-                ("act", ctypes.c_int32)]
+                ("act", ctypes.c_int32), ("qkv_silu", ctypes.c_int32)]
 
 
 def mixers_so_path() -> str:
@@ -395,6 +395,14 @@ def mixers() -> ctypes.CDLL:
         L.gbxm_conv_tail_update.argtypes = [p, i64, p, p, i32, i32, i32, i32, p]
         L.gbxm_state_scan.argtypes = [p, i64, p, p, p, i32, i64, i32, i32, i32, i32, i32, p]
         L.gbxm_head_norm_gate.argtypes = [p, p, i64, p, p, i64, i32, i32, f32, i32, i32, p]
+        L.gbxm_embed_hashed_pair.argtypes = [p, p, p, p, p, p, p, i64, i32, i64, i64, i64, i32, p]
+        L.gbxm_norm_token_shift.argtypes = [p, p, p, p, p, p, p, i64, i32, f32, i32, p]
+        L.gbxm_branch_norm_add_norm.argtypes = [p, p, p, p, p, p, p, i64, i32, i32, f32, i32, p]
+        L.gbxm_normed_pair_mean.argtypes = [p, p, p, p, p, i64, i32, f32, i32, p]
+        L.gbxm_gate_mul.argtypes = [p, i64, p, i64, p, i64, i32, i32, i32, p]
+        L.gbxm_causal_conv_rows.argtypes = [p, i64, p, p, p, p, p, p, i64, i32, i32, i32, p]
+        L.gbxm_block_gate_logits.argtypes = [p, p, p, p, i64, i32, i32, i32, i32, p]
+        L.gbxm_gated_lru_scan.argtypes = [p, p, i64, i64, p, p, i64, p, p, p, i32, i64, i32, i32, f32, i32, p]
         _mlib = L
     return _mlib
 

@@ -47,14 +47,16 @@ template <bool FAST> __device__ __forceinline__ float sigmoid_(float x) {
 template <bool FAST> __device__ __forceinline__ float tanh_(float x) {
   if constexpr (FAST) { const float e = __expf(2.f * x); return 1.f - __fdividef(2.f, e + 1.f); } else return tanhf(x);
 }
-// Gated activations of feed-forwards (GBXM_GLU_*): silu(g) u, or the clamped form g' sigmoid(alpha g') (u' + 1) with g' = min(g, limit),
-// u' = clamp(u, -limit, limit).
+// Gated activations of feed-forwards (GBXM_GLU_*): silu(g) u, gelu(g) u in the tanh form, sigmoid(g) u, or the clamped form
+// g' sigmoid(alpha g') (u' + 1) with g' = min(g, limit), u' = clamp(u, -limit, limit).
 template <bool FAST> __device__ __forceinline__ float glu_act(float g, float u, int kind, float limit, float alpha) {
   if (kind == GBXM_GLU_CLAMPED_SWISH) {
     g = fminf(g, limit);
     u = fminf(fmaxf(u, -limit), limit);
     return g * sigmoid_<FAST>(alpha * g) * (u + 1.f);
   }
+  if (kind == GBXM_GLU_GELU_TANH) return 0.5f * g * (1.f + tanh_<FAST>(0.7978845608028654f * (g + 0.044715f * g * g * g))) * u;
+  if (kind == GBXM_GLU_SIGMOID) return sigmoid_<FAST>(g) * u;
   return g * sigmoid_<FAST>(g) * u;
 }
 template <bool FAST> __device__ __forceinline__ float log1p_(float x) { if constexpr (FAST) return __logf(1.f + x); else return log1pf(x); }

@@ -324,6 +324,15 @@ __global__ __launch_bounds__(NT) void rotate_norm_kernel(T* __restrict__ rows, i
     if (live)
       for (int c = lane; c < sg.head_dim; c += 64) in[c] = to_f32(p[c]);
     __syncthreads();
+    if (sg.norm >= 3) {                             // norm before the rotation: the staged head is replaced by its normed image
+      if (live) {
+        float s0 = 0.f;
+        for (int c = lane; c < sg.head_dim; c += 64) s0 += in[c] * in[c];
+        const float r0 = 1.f / sqrtf(wave_sum(s0) / sg.head_dim + eps);
+        for (int c = lane; c < sg.head_dim; c += 64) in[c] = in[c] * r0 * (sg.norm == 4 ? sg.weight[c] : 1.f);
+      }
+      __syncthreads();
+    }
     if (!live) continue;
     float ss = 0.f;
     for (int c = lane; c < sg.head_dim; c += 64) {
@@ -342,7 +351,7 @@ __global__ __launch_bounds__(NT) void rotate_norm_kernel(T* __restrict__ rows, i
       ss += v * v;
     }
     float r = 1.f;
-    if (sg.norm) r = 1.f / sqrtf(wave_sum(ss) / sg.head_dim + eps);
+    if (sg.norm == 1 || sg.norm == 2) r = 1.f / sqrtf(wave_sum(ss) / sg.head_dim + eps);
     for (int c = lane; c < sg.head_dim; c += 64) {
       float v = turned[c] * r;
       if (sg.norm == 2) v *= sg.weight[c];
@@ -589,8 +598,8 @@ int gbxm_rotate_norm_heads(void* rows, int64_t T_, int64_t row_stride, const int
   for (int i = 0; i < n_segs; ++i) {
     const gbxm_head_segment& g = segs[i];
     if (g.offset < 0 || g.heads < 1 || g.head_dim < 1 || g.offset + static_cast<int64_t>(g.heads) * g.head_dim > row_stride || g.rot_dims < 0 ||
-        g.rot_dims % 2 || g.rot_offset < 0 || g.rot_offset + g.rot_dims > g.head_dim || (g.rot_dims && !g.freq) || g.norm < 0 || g.norm > 2 ||
-        (g.norm == 2 && !g.weight))
+        g.rot_dims % 2 || g.rot_offset < 0 || g.rot_offset + g.rot_dims > g.head_dim || (g.rot_dims && !g.freq) || g.norm < 0 || g.norm > 4 ||
+        ((g.norm == 2 || g.norm == 4) && !g.weight))
       return fail(GBXM_ERR_INVALID, "rotate_norm_heads: segment %d does not fit its rows", i);
     sg.s[i] = g;
     max_dim = std::max(max_dim, g.head_dim);

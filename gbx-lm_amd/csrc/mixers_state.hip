@@ -36,7 +36,7 @@ __global__ __launch_bounds__(NT) void recurrent_prep_kernel(gbxm_recurrent_prep_
   float* out = p.out + t * p.out_stride;
   // channel c of q | k | v after the convolution and silu (or as projected, without a convolution; `plain`: its offset in the row)
   auto value = [&](int c, int plain) {
-    if (!cw) return to_f32(yr[plain]);
+    if (!cw) { const float x = to_f32(yr[plain]); return p.qkv_silu ? x * sigmoid_<FAST>(x) : x; }
     float acc = 0.f;
     for (int j = 0; j < p.taps; ++j) {
       const int src = pos - (p.taps - 1) + j;
@@ -71,7 +71,9 @@ __global__ __launch_bounds__(NT) void recurrent_prep_kernel(gbxm_recurrent_prep_
   }
   for (int c = gthread; c < nv; c += n_threads) out[2 * nq + c] = value(2 * nq + c, p.off_v + c);
   const T* ar = static_cast<const T*>(p.a) + t * p.a_stride;
-  for (int c = gthread; c < nd; c += n_threads) {
+  if (!p.a) {                               // no decay projection: the head's constant
+    for (int c = gthread; c < nd; c += n_threads) out[2 * nq + nv + c] = p.decay_rate[c / p.dk];
+  } else for (int c = gthread; c < nd; c += n_threads) {
     const float z = p.sign * (to_f32(ar[c]) + p.decay_bias[c]);
     const float sp = z > 20.f ? z : log1p_<FAST>(exp_<FAST>(z));
     out[2 * nq + nv + c] = exp_<FAST>(-p.decay_rate[c / p.dk] * sp);
@@ -265,7 +267,7 @@ using namespace gbxm;
 extern "C" {
 
 int gbxm_recurrent_prepare(const gbxm_recurrent_prep_args* a, void* stream) {
-  if (!a || !act_ok(a->act) || !a->y || !a->a || !a->decay_bias || !a->decay_rate || !a->seq || !a->tok || !a->out || a->T < 0 || a->H < 1 || a->G < 1 ||
+  if (!a || !act_ok(a->act) || !a->y || (a->a && !a->decay_bias) || !a->decay_rate || !a->seq || !a->tok || !a->out || a->T < 0 || a->H < 1 || a->G < 1 ||
       a->H % a->G || a->dk < 1 || a->dv < 1 || a->off_q < 0 || a->off_k < 0 || a->off_v < 0)
     return fail(GBXM_ERR_INVALID, "recurrent_prepare: bad argument");
   const int nq = a->G * a->dk, nv = a->H * a->dv, C = 2 * nq + nv;

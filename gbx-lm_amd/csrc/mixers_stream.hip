@@ -220,7 +220,7 @@ int gbxm_hyper_step(float* X, const void* y, const float* y_mix, const float* mi
 }
 
 int gbxm_glu(const void* gu, int64_t gu_stride, void* out, int64_t T_, int32_t F, int32_t kind, float limit, float alpha, int32_t act, void* stream) {
-  if (!act_ok(act) || !gu || !out || F <= 0 || gu_stride < 2 * F || T_ < 0 || (kind != GBXM_GLU_SILU && kind != GBXM_GLU_CLAMPED_SWISH))
+  if (!act_ok(act) || !gu || !out || F <= 0 || gu_stride < 2 * F || T_ < 0 || kind < GBXM_GLU_SILU || kind > GBXM_GLU_SIGMOID)
     return fail(GBXM_ERR_INVALID, "glu: bad argument");
   if (T_ == 0) return GBXM_OK;
   if (T_ > 65535) {                       // rows ride on grid.y: long steps go in slices

@@ -98,7 +98,7 @@ def route_topk(h: torch.Tensor, router: torch.Tensor, top: int, renormalize: boo
     return idx, w
 
 
-_GLU = {"silu": 1, "clamped_swish": 2}
+_GLU = {"silu": 1, "clamped_swish": 2, "gelu_tanh": 3, "sigmoid": 4}
 
 
 def expert_glu(h: torch.Tensor, gate_up: torch.Tensor, down: torch.Tensor, idx: torch.Tensor, activation: str = "silu",
@@ -219,7 +219,7 @@ def rotate_norm_heads_(rows: torch.Tensor, positions: torch.Tensor, segments, ep
         if s.weight is not None and s.weight.numel() != s.head_dim:
             raise ValueError("rotate_norm_heads_: one weight per channel of the head")
         c.offset, c.heads, c.head_dim, c.rot_offset, c.rot_dims = s.offset, s.heads, s.head_dim, s.rot_offset, s.rot_dims
-        c.interleaved, c.norm, c.mult, c.sign = int(s.interleaved), s.norm, s.mult, s.sign
+        c.interleaved, c.norm, c.mult, c.sign = int(s.interleaved), s.norm + (2 if (s.norm and getattr(s, "norm_first", False)) else 0), s.mult, s.sign
         c.freq = _f32(s.freq, "freq").data_ptr() if s.rot_dims else None
         c.weight = _f32(s.weight, "weight").data_ptr() if s.weight is not None else None
     _lib.check_mixers(_lib.mixers().gbxm_rotate_norm_heads(rows.data_ptr(), rows.shape[0], rows.stride(0), positions.data_ptr(), positions.stride(0),
@@ -356,19 +356,21 @@ def route_sigmoid_groups(h: torch.Tensor, router: torch.Tensor, correction: torc
 
 
 # ------------------------------------------------------------------------------- recurrent mixers (models/recurrent_mixers.py)
-def recurrent_prepare(y: torch.Tensor, a: torch.Tensor, lay, decay_bias: torch.Tensor, decay_rate: torch.Tensor, sign: float,
-                      conv: Optional[torch.Tensor], cache, batch, unit: bool, q_scale: float) -> torch.Tensor:
+def recurrent_prepare(y: torch.Tensor, a: Optional[torch.Tensor], lay, decay_bias: Optional[torch.Tensor], decay_rate: torch.Tensor, sign: float,
+                      conv: Optional[torch.Tensor], cache, batch, unit: bool, q_scale: float, qkv_silu: bool = False) -> torch.Tensor:
     act = _act(y, "y")
     t = y.shape[0]
-    if y.dim() != 2 or y.stride(1) != 1 or a.dim() != 2 or a.stride(1) != 1 or a.dtype != y.dtype or a.shape != (t, lay.nd) or t != batch.total:
+    if y.dim() != 2 or y.stride(1) != 1 or t != batch.total or (a is not None and (a.dim() != 2 or a.stride(1) != 1 or a.dtype != y.dtype or a.shape != (t, lay.nd))):
         raise ValueError("recurrent_prepare: projection rows do not fit the step")
     if max(lay.off_q + lay.nq, lay.off_k + lay.nq, lay.off_v + lay.nv, lay.off_beta + lay.heads) > y.shape[1]:
         raise ValueError("recurrent_prepare: the layout ends outside the rows")
-    if decay_bias.numel() != lay.nd or decay_rate.numel() != lay.heads:
+    if (a is not None and decay_bias.numel() != lay.nd) or decay_rate.numel() != lay.heads:
         raise ValueError("recurrent_prepare: one decay bias per head and key channel, one rate per head")
     out = torch.empty((t, lay.out_width), dtype=torch.float32, device=y.device)
     p = _lib.RecurrentPrepArgs()
-    p.y, p.y_stride, p.a, p.a_stride = y.data_ptr(), y.stride(0), a.data_ptr(), a.stride(0)
+    p.y, p.y_stride = y.data_ptr(), y.stride(0)
+    p.a, p.a_stride = (a.data_ptr(), a.stride(0)) if a is not None else (None, 0)
+    p.qkv_silu = int(bool(qkv_silu))
     p.conv = p.tail = None
     p.taps = 0
     if conv is not None:
@@ -381,7 +383,8 @@ def recurrent_prepare(y: torch.Tensor, a: torch.Tensor, lay, decay_bias: torch.T
             if tail is None or tail.dtype != y.dtype or tuple(tail.shape[1:]) != (p.taps - 1, c) or tail.shape[0] <= max(batch.slot) or not tail.is_contiguous():
                 raise ValueError("recurrent_prepare: the cache's tails do not fit the convolution or the step's slots")
             p.tail = tail.data_ptr()
-    p.decay_bias, p.decay_rate = _f32(decay_bias, "decay_bias").data_ptr(), _f32(decay_rate, "decay_rate").data_ptr()
+    p.decay_bias = _f32(decay_bias, "decay_bias").data_ptr() if a is not None else None
+    p.decay_rate = _f32(decay_rate, "decay_rate").data_ptr()
     p.seq, p.tok, p.out, p.out_stride, p.T = batch.seq.data_ptr(), batch.tok.data_ptr(), out.data_ptr(), out.stride(0), t
     p.H, p.G, p.dk, p.dv = lay.heads, lay.groups, lay.dk, lay.dv
     p.off_q, p.off_k, p.off_v, p.off_beta = lay.off_q, lay.off_k, lay.off_v, lay.off_beta
@@ -421,4 +424,130 @@ def head_norm_gate(o: torch.Tensor, gate: torch.Tensor, weight: torch.Tensor, he
     out = torch.empty((t, n), dtype=gate.dtype, device=o.device)
     _lib.check_mixers(_lib.mixers().gbxm_head_norm_gate(o.data_ptr(), gate.data_ptr(), gate.stride(0), _f32(weight, "weight").data_ptr(), out.data_ptr(),
                                                        t, heads, n // heads, float(eps), int(kind), act, _stream(o.device)))
+    return out
+
+
+# ------------------------------------------------------------------------------- sandwich-norm layers, token shift, hashed pair embedding
+def embed_hashed_pair(table: torch.Tensor, pair: torch.Tensor, tokens: torch.Tensor, batch, state: torch.Tensor, buckets: int, mul_prev: int,
+                      mul_cur: int) -> torch.Tensor:
+    """models/embedding.py:HashedPairEmbedding as one launch: fp32 [T, W]; ``state`` int64 [slots, 1] holds each sequence's last token."""
+    act = _act(table, "table")
+    t, w = tokens.numel(), table.shape[1]
+    if tokens.dtype != torch.int64 or not tokens.is_contiguous() or t != batch.total:
+        raise ValueError("embed_hashed_pair: the step's tokens as contiguous int64")
+    if pair.dtype != table.dtype or tuple(pair.shape) != (buckets + 1, w) or not (pair.is_contiguous() and table.is_contiguous()):
+        raise ValueError("embed_hashed_pair: the pair table is [buckets + 1, width] in the embedding's dtype")
+    if state.dtype != torch.int64 or not state.is_contiguous() or state.shape[0] <= max(batch.slot):
+        raise ValueError("embed_hashed_pair: one int64 per slot")
+    x = torch.empty((t, w), dtype=torch.float32, device=table.device)
+    _lib.check_mixers(_lib.mixers().gbxm_embed_hashed_pair(table.data_ptr(), pair.data_ptr(), tokens.data_ptr(), state.data_ptr(), batch.seq.data_ptr(),
+                                                          batch.tok.data_ptr(), x.data_ptr(), t, w, int(buckets), int(mul_prev), int(mul_cur), act,
+                                                          _stream(table.device)))
+    return x
+
+
+def norm_token_shift(x: torch.Tensor, w: torch.Tensor, eps: float, shift: torch.Tensor, state: torch.Tensor, batch, act_dtype: torch.dtype) -> torch.Tensor:
+    _f32(x, "x")
+    if not x.is_cuda or x.dim() != 2 or x.shape[0] != batch.total or w.numel() != x.shape[1] or shift.numel() != x.shape[1]:
+        raise ValueError("norm_token_shift: fp32 device rows of the step, one weight and one shift per channel")
+    if state.dtype != torch.float32 or not state.is_contiguous() or state.shape[1] != x.shape[1] or state.shape[0] <= max(batch.slot):
+        raise ValueError("norm_token_shift: one fp32 row per slot")
+    h = torch.empty(x.shape, dtype=act_dtype, device=x.device)
+    _lib.check_mixers(_lib.mixers().gbxm_norm_token_shift(x.data_ptr(), _f32(w, "w").data_ptr(), _f32(shift, "shift").data_ptr(), state.data_ptr(),
+                                                         batch.seq.data_ptr(), batch.tok.data_ptr(), h.data_ptr(), x.shape[0], x.shape[1], float(eps),
+                                                         _DT[act_dtype], _stream(x.device)))
+    return h
+
+
+def branch_norm_add_norm_(x: torch.Tensor, branch: torch.Tensor, mix: Optional[torch.Tensor], extra: Optional[torch.Tensor], w: torch.Tensor, eps: float,
+                          next_w: Optional[torch.Tensor], act_dtype: torch.dtype) -> Optional[torch.Tensor]:
+    act = _act(branch, "branch")
+    _f32(x, "x")
+    t, width = x.shape
+    top = 1 if mix is None else mix.shape[-1]
+    branch = branch.contiguous()
+    if branch.dtype != act_dtype or branch.numel() != t * top * width or w.numel() != width:
+        raise ValueError("branch_norm_add_norm_: the branch is [T, (top,) W] in the activation dtype")
+    if extra is not None and (extra.dtype != act_dtype or extra.shape != (t, width) or not extra.is_contiguous()):
+        raise ValueError("branch_norm_add_norm_: the extra branch is contiguous [T, W] in the activation dtype")
+    h = None if next_w is None else torch.empty((t, width), dtype=act_dtype, device=x.device)
+    _lib.check_mixers(_lib.mixers().gbxm_branch_norm_add_norm(
+        x.data_ptr(), branch.data_ptr(), None if mix is None else _f32(mix, "mix").data_ptr(), None if extra is None else extra.data_ptr(),
+        _f32(w, "w").data_ptr(), None if next_w is None else _f32(next_w, "next_w").data_ptr(), None if h is None else h.data_ptr(), t, width, top,
+        float(eps), act, _stream(x.device)))
+    return h
+
+
+def normed_pair_mean(a: torch.Tensor, b: torch.Tensor, wa: torch.Tensor, wb: torch.Tensor, eps: float) -> torch.Tensor:
+    act = _act(a, "a")
+    if a.dim() != 2 or b.shape != a.shape or b.dtype != a.dtype or not (a.is_contiguous() and b.is_contiguous()) or wa.numel() != a.shape[1] or wb.numel() != a.shape[1]:
+        raise ValueError("normed_pair_mean: two contiguous [T, W] branches of one dtype, a weight per channel each")
+    out = torch.empty_like(a)
+    _lib.check_mixers(_lib.mixers().gbxm_normed_pair_mean(a.data_ptr(), b.data_ptr(), _f32(wa, "wa").data_ptr(), _f32(wb, "wb").data_ptr(), out.data_ptr(),
+                                                         a.shape[0], a.shape[1], float(eps), act, _stream(a.device)))
+    return out
+
+
+def gate_mul(gate: torch.Tensor, up: torch.Tensor, kind: str) -> torch.Tensor:
+    act = _act(up, "up")
+    if gate.dim() != 2 or gate.shape != up.shape or gate.dtype != up.dtype or gate.stride(1) != 1 or up.stride(1) != 1:
+        raise ValueError("gate_mul: rows [T, F] of one dtype with unit inner stride")
+    out = torch.empty(up.shape, dtype=up.dtype, device=up.device)
+    _lib.check_mixers(_lib.mixers().gbxm_gate_mul(gate.data_ptr(), gate.stride(0), up.data_ptr(), up.stride(0), out.data_ptr(), up.shape[0], up.shape[1],
+                                                 _GLU[kind], act, _stream(up.device)))
+    return out
+
+
+# ------------------------------------------------------------------------------- gated linear recurrent unit (models/gated_lru.py)
+def causal_conv_rows(x: torch.Tensor, conv: torch.Tensor, bias: Optional[torch.Tensor], cache, batch) -> torch.Tensor:
+    act = _act(x, "x")
+    t, c = x.shape
+    taps = conv.shape[1]
+    if x.stride(1) != 1 or t != batch.total or conv.shape[0] != c or conv.dtype != x.dtype or not conv.is_contiguous():
+        raise ValueError("causal_conv_rows: rows of the step, taps [C, taps] in the rows' dtype")
+    tail = cache.tail if taps > 1 else None
+    if taps > 1 and (tail is None or tail.dtype != x.dtype or tuple(tail.shape[1:]) != (taps - 1, c) or tail.shape[0] <= max(batch.slot) or not tail.is_contiguous()):
+        raise ValueError("causal_conv_rows: the cache's tails do not fit the convolution or the step's slots")
+    out = torch.empty((t, c), dtype=torch.float32, device=x.device)
+    _lib.check_mixers(_lib.mixers().gbxm_causal_conv_rows(x.data_ptr(), x.stride(0), conv.data_ptr(), None if bias is None else _f32(bias, "bias").data_ptr(),
+                                                         None if tail is None else tail.data_ptr(), batch.seq.data_ptr(), batch.tok.data_ptr(), out.data_ptr(),
+                                                         t, c, taps, act, _stream(x.device)))
+    return out
+
+
+def block_gate_logits(u: torch.Tensor, w: torch.Tensor, b: torch.Tensor, w_t_f32: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """fp32 logits, element (t, block, o) of the returned tensor (which may be a permuted view).  Few rows: one HIP launch; prompt-sized
+    steps: a batched fp32 product of the vendor library over ``w_t_f32`` [blocks, bs, n_out], the fp32 image of ``w`` transposed."""
+    act = _act(w, "w")
+    _f32(u, "u")
+    blocks, n_out, bs = w.shape
+    t = u.shape[0]
+    if u.shape[1] != blocks * bs or not w.is_contiguous() or tuple(b.shape) != (blocks, n_out):
+        raise ValueError("block_gate_logits: operands do not fit")
+    if t <= 16 or w_t_f32 is None:
+        out = torch.empty((t, blocks, n_out), dtype=torch.float32, device=u.device)
+        _lib.check_mixers(_lib.mixers().gbxm_block_gate_logits(u.data_ptr(), w.data_ptr(), _f32(b, "b").data_ptr(), out.data_ptr(), t, blocks, bs, n_out, act,
+                                                              _stream(u.device)))
+        return out
+    if w_t_f32.dtype != torch.float32 or tuple(w_t_f32.shape) != (blocks, bs, n_out):
+        raise ValueError("block_gate_logits: the fp32 image is [blocks, bs, n_out]")
+    return torch.baddbmm(b.unsqueeze(1), u.view(t, blocks, bs).transpose(0, 1), w_t_f32).transpose(0, 1)
+
+
+def gated_lru_scan(u: torch.Tensor, logits: torch.Tensor, lam_sp: torch.Tensor, y: torch.Tensor, rate: float, cache, batch) -> torch.Tensor:
+    act = _act(y, "y")
+    _f32(u, "u")
+    t, c = u.shape
+    blocks, bs = logits.shape[1], logits.shape[2] // 2
+    state = cache.state
+    if t != batch.total or logits.dtype != torch.float32 or logits.shape != (t, blocks, 2 * bs) or blocks * bs != c or logits.stride(2) != 1:
+        raise ValueError("gated_lru_scan: logits [T, blocks, 2 * block size] in fp32")
+    if y.shape != (t, c) or y.stride(1) != 1 or lam_sp.numel() != c:
+        raise ValueError("gated_lru_scan: the other branch's rows and one rate per channel")
+    if state is None or state.dtype != torch.float32 or state.numel() != state.shape[0] * c or state.shape[0] <= max(batch.slot) or not state.is_contiguous():
+        raise ValueError("gated_lru_scan: the cache's states do not fit the unit or the step's slots")
+    out = torch.empty((t, c), dtype=y.dtype, device=y.device)
+    _lib.check_mixers(_lib.mixers().gbxm_gated_lru_scan(u.data_ptr(), logits.data_ptr(), logits.stride(0), logits.stride(1), _f32(lam_sp, "lam_sp").data_ptr(),
+                                                       y.data_ptr(), y.stride(0), state.data_ptr(), out.data_ptr(), batch.seq.data_ptr(), len(batch.slot), t, c, bs,
+                                                       float(rate), act, _stream(y.device)))
     return out

@@ -55,12 +55,13 @@ def causal_conv_rows(x: torch.Tensor, conv: torch.Tensor, bias: Optional[torch.T
     return out
 
 
-def block_gate_logits(u: torch.Tensor, w: torch.Tensor, b: torch.Tensor) -> torch.Tensor:
+def block_gate_logits(u: torch.Tensor, w: torch.Tensor, b: torch.Tensor, w_t_f32: Optional[torch.Tensor] = None) -> torch.Tensor:
     """u fp32 [T, C], w [blocks, 2 * bs, bs] (rows: the recurrence gate's matrix over the input gate's, each [out, in]; activation
-    dtype), b fp32 [blocks, 2 * bs] -> fp32 logits [T, blocks, 2 * bs]; products and sums in fp32."""
+    dtype), b fp32 [blocks, 2 * bs] -> fp32 logits [T, blocks, 2 * bs]; products and sums in fp32.  ``w_t_f32`` [blocks, bs, 2 * bs]:
+    the fp32 image of w transposed, which prompt-sized GPU steps multiply with (a batched vendor product)."""
     if u.is_cuda:
         from .. import mixer_ops as M
-        return M.block_gate_logits(u, w, b)
+        return M.block_gate_logits(u, w, b, w_t_f32)
     blocks, two_bs, bs = w.shape
     ub = u.view(u.shape[0], blocks, bs)
     return torch.einsum("tbi,boi->tbo", ub, w.float()) + b.float()[None]
@@ -108,8 +109,15 @@ class GatedLRUBlock(nn.Module):
         self.register_buffer("gates", torch.zeros((blocks, 2 * bs, bs)))                   # activation dtype
         self.register_buffer("gates_bias", torch.zeros((blocks, 2 * bs), dtype=torch.float32))
         self.register_buffer("lam_sp", torch.zeros(lru_width, dtype=torch.float32))        # softplus(lam), formed once in fp32
+        self._gates_t = None                                                               # fp32 transposed image, formed at the first long GPU step
         for p in self.parameters():
             p.requires_grad_(False)
+
+    def _gates_f32_t(self) -> torch.Tensor:
+        g = self.gates
+        if self._gates_t is None or self._gates_t.device != g.device or self._gates_src != (g.data_ptr(), g._version):
+            self._gates_t, self._gates_src = g.float().transpose(1, 2).contiguous(), (g.data_ptr(), g._version)
+        return self._gates_t
 
     def make_cache(self, slots) -> SlotStateCache:
         return SlotStateCache(1, 1, self.lru_width, self.lru_width, self.taps, slots)
@@ -121,5 +129,5 @@ class GatedLRUBlock(nn.Module):
         u = causal_conv_rows(xy[:, :c], self.conv, self.conv_bias, cache, batch)
         if self.taps > 1:
             conv_tail_update(xy, c, cache, batch)
-        logits = block_gate_logits(u, self.gates, self.gates_bias)
+        logits = block_gate_logits(u, self.gates, self.gates_bias, self._gates_f32_t() if (u.is_cuda and u.shape[0] > 16) else None)
         return F.linear(gated_lru_scan(u, logits, self.lam_sp, xy[:, c:], self.rate, cache, batch), self.o.weight)

@@ -92,7 +92,8 @@ int gbxm_activate(void* z, int64_t n, int32_t kind, int32_t act, void* stream);
 
 /* A run of `heads` heads of `head_dim` channels at `offset` of every row.  Channels [rot_offset, rot_offset + rot_dims) of each head
  * turn by sign * position * freq[i] (pairs i, i + rot_dims/2; or 2i, 2i+1 when interleaved), cos and sin times mult; then the head
- * is scaled to unit root mean square (norm 1) or RMS-normalised with `weight` [head_dim] (norm 2).  All in fp32, in place. */
+ * is scaled to unit root mean square (norm 1) or RMS-normalised with `weight` [head_dim] (norm 2); norm 3 / 4: the same two norms
+ * BEFORE the rotation.  All in fp32, in place. */
 typedef struct {
   int32_t offset, heads, head_dim, rot_offset, rot_dims, interleaved, norm;
   float mult, sign;
@@ -151,6 +152,8 @@ int gbxm_hyper_step(float* X, const void* y, const float* y_mix, const float* mi
  * kind 1: g sigmoid(g) u;  kind 2: g' = min(g, limit), u' = clamp(u, -limit, limit), g' sigmoid(alpha g') (u' + 1). */
 #define GBXM_GLU_SILU 1
 #define GBXM_GLU_CLAMPED_SWISH 2
+#define GBXM_GLU_GELU_TANH 3      /* gelu(g) u, gelu in its tanh form */
+#define GBXM_GLU_SIGMOID 4        /* sigmoid(g) u */
 int gbxm_glu(const void* gu, int64_t gu_stride, void* out, int64_t T, int32_t F, int32_t kind, float limit, float alpha, int32_t act, void* stream);
 /* Router decisions from fp32 logits [T][E]: s = sigmoid(logit), choice score c = s + correction; with n_groups > 0 the experts form
  * n_groups equal groups of neighbours, a group's score is the sum of its two largest c, and only experts of the keep_groups best
@@ -168,7 +171,7 @@ int gbxm_expert_glu_act(const void* h, const void* gate_up, const void* down, co
  * off_beta (< 0: none); `a` rows [T][H*dk] are the decay projection.  With conv (rows [2 G dk + H dv][taps], q | k | v must be adjacent
  * from off_q on): c[t] = silu(sum_j conv[c][j] in[t - (taps-1) + j]), inputs before the step from tail [slots][taps-1][C] (oldest
  * first), zeros before the sequence.  unit: q, k heads / sqrt(sum sq + 1e-6).  out row: q * q_scale | k | v | decay | beta with
- * decay = exp(-rate[h] * softplus(sign * (a + bias))), beta = sigmoid(.). */
+ * decay = exp(-rate[h] * softplus(sign * (a + bias))), beta = sigmoid(.).  `a` null (then decay_bias may be null): decay = rate[h]. */
 typedef struct {
   const void* y;    int64_t y_stride;
   const void* a;    int64_t a_stride;
@@ -183,6 +186,7 @@ typedef struct {
   int32_t H, G, dk, dv, off_q, off_k, off_v, off_beta, taps, unit;
   float sign, q_scale;
   int32_t act;
+  int32_t qkv_silu;             /* without conv: q | k | v pass silu */
 } gbxm_recurrent_prep_args;
 int gbxm_recurrent_prepare(const gbxm_recurrent_prep_args* a, void* stream);
 /* tail[slot] <- the last taps-1 inputs (channels [0, C) of y) of every sequence of the step; older ones shift out. */
@@ -196,6 +200,44 @@ int gbxm_state_scan(const float* r, int64_t r_stride, float* state, float* out, 
 /* out[t][h][c] = o[t][h][c] / sqrt(mean_c o^2 + eps) * w[c] * gate(g[t][h][c]); gate kind 1 silu, 2 sigmoid; o fp32, g / out activation dtype. */
 int gbxm_head_norm_gate(const float* o, const void* gate, int64_t gate_stride, const float* w, void* out, int64_t T, int32_t H, int32_t dv,
                         float eps, int32_t kind, int32_t act, void* stream);
+
+/* ---- sandwich-norm layers, token shift, hashed pair embedding (gbx-lm_amd/models/residual.py, models/embedding.py) ---- */
+
+/* x[t] = table[token[t]] + pair[row], row = (prev * mul_prev + token * mul_cur) mod buckets, or `buckets` for a sequence's first token;
+ * prev = the row before in the step, or state[slot] (int64) for the step's first row.  state[slot] <- the sequence's last token. */
+int gbxm_embed_hashed_pair(const void* table, const void* pair, const int64_t* tokens, int64_t* state, const int32_t* seq, const int32_t* tok,
+                           float* x, int64_t T, int32_t width, int64_t buckets, int64_t mul_prev, int64_t mul_cur, int32_t act, void* stream);
+/* n[t] = rms_norm(x[t]) * w;  h[t] = n[t] + (n[t-1] - n[t]) * shift in the activation dtype; n[t-1] of a step's first row is
+ * state[slot] (fp32 [slots][width]) or zero at position 0; state[slot] <- n of the sequence's last row. */
+int gbxm_norm_token_shift(const float* x, const float* w, const float* shift, float* state, const int32_t* seq, const int32_t* tok, void* h,
+                          int64_t T, int32_t width, float eps, int32_t act, void* stream);
+/* z = branch[t] (top == 1) or sum_k mix[t][k] branch[t][k], plus extra[t] if given;  x[t] += rms_norm(z) * w;  with next_w:
+ * h[t] = rms_norm(x[t]) * next_w in the activation dtype. */
+int gbxm_branch_norm_add_norm(float* x, const void* branch, const float* mix, const void* extra, const float* w, const float* next_w, void* h,
+                              int64_t T, int32_t width, int32_t top, float eps, int32_t act, void* stream);
+/* out[t] = (rms_norm(a[t]) * wa + rms_norm(b[t]) * wb) / 2, rows of the activation dtype. */
+int gbxm_normed_pair_mean(const void* a, const void* b, const float* wa, const float* wb, void* out, int64_t T, int32_t width, float eps,
+                          int32_t act, void* stream);
+/* out[t][f] = act(gate[t][f]) * up[t][f] (GBXM_GLU_SILU / GELU_TANH / SIGMOID), row strides in elements, out rows contiguous. */
+int gbxm_gate_mul(const void* gate, int64_t gate_stride, const void* up, int64_t up_stride, void* out, int64_t T, int32_t F, int32_t kind,
+                  int32_t act, void* stream);
+
+/* ---- gated linear recurrent unit (gbx-lm_amd/models/gated_lru.py) ---- */
+
+/* out[t][c] = bias[c] + sum_j conv[c][j] x[t - (taps-1) + j][c] in fp32; inputs before the step from tail [slots][taps-1][C] (oldest
+ * first; the activation dtype), zeros before the sequence.  bias may be null. */
+int gbxm_causal_conv_rows(const void* x, int64_t x_stride, const void* conv, const float* bias, const void* tail, const int32_t* seq,
+                          const int32_t* tok, float* out, int64_t T, int32_t C, int32_t taps, int32_t act, void* stream);
+/* logits[t][b][o] = bias[b][o] + sum_i w[b][o][i] u[t][b * bs + i], o < n_out; u fp32 [T][blocks * bs], w [blocks][n_out][bs] in the
+ * activation dtype, fp32 sums in a fixed order. */
+int gbxm_block_gate_logits(const float* u, const void* w, const float* bias, float* logits, int64_t T, int32_t blocks, int32_t bs, int32_t n_out,
+                           int32_t act, void* stream);
+/* logits: element (t, b, o) at t * lg_t + b * lg_b + o (floats).  Per channel c of block b = c / bs:  r = sigmoid(logits[t][b][c % bs]),
+ * i = sigmoid(logits[t][b][bs + c % bs]),
+ * a = exp(-rate * r * lam_sp[c]), S <- a S + sqrt(1 - a^2) i u[t][c] over each sequence's rows from state[slot][c] (zero at position
+ * 0; written back); out[t][c] = S * gelu_tanh(y[t][c]) in the activation dtype. */
+int gbxm_gated_lru_scan(const float* u, const float* logits, int64_t lg_t, int64_t lg_b, const float* lam_sp, const void* y, int64_t y_stride, float* state, void* out,
+                        const int32_t* seq, int32_t B, int64_t T, int32_t C, int32_t bs, float rate, int32_t act, void* stream);
 
 #ifdef __cplusplus
 }
