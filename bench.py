@@ -699,9 +699,85 @@ def tugolix_bench(args):
     print(json.dumps({"metric": "tugolix_throughput", "unit": "tokens/s", "dtype": "bf16", "data": "synthetic", "sizes": out}))
 
 
+LARUZEN_SIZES = {
+    # name: Laruzen geometry (layers: gated linear attention, lightning attention, the parallel pair of windowed sink attention and a
+    # gated linear recurrent unit, gated linear attention; dense feed-forward in the first layer, routed experts with a shared one in the
+    # others) and, from it, the Tugolix (the closest existing model: dense bf16 decoder over ragged steps with recurrent mixers of the same
+    # scan and routed experts) of equal width, layer count, experts and gated-linear-attention geometry
+    "small": dict(width=1024, gla=dict(heads=4, dim=128, vdim=256, tau=16.0), lightning=dict(heads=8, dim=128, vdim=128),
+                  left=dict(heads=16, kv_heads=4, dim=64, vdim=64, window=1024), right=dict(width=1024, blocks=8, conv=4), ff=4096,
+                  moe=dict(experts=32, top=4, ff=512, shared=1024), pattern="glpg"),
+    "a3b-like": dict(width=2048, gla=dict(heads=8, dim=128, vdim=256, tau=16.0), lightning=dict(heads=16, dim=128, vdim=128),
+                     left=dict(heads=16, kv_heads=4, dim=128, vdim=128, window=4096), right=dict(width=2560, blocks=10, conv=4), ff=8192,
+                     moe=dict(experts=128, top=8, ff=768, shared=1536), pattern="glpg"),
+    "recurrent": dict(width=2048, gla=dict(heads=8, dim=128, vdim=256, tau=16.0), lightning=dict(heads=16, dim=128, vdim=128),
+                      left=dict(heads=16, kv_heads=2, dim=128, vdim=128, window=2048), right=dict(width=2048, blocks=16, conv=4), ff=8192,
+                      moe=dict(experts=64, top=4, ff=1024, shared=1024), pattern="lplp"),
+}
+
+
+def laruzen_bench(args):
+    """``--design laruzen``: prefill and decode throughput of Laruzen at layer sizes of real models (random weights, bf16), beside
+    Tugolix of equal width, layer count, routed experts and gated-linear-attention geometry.  One JSON line; the default workload of
+    this file is untouched."""
+    from gbx_lm_amd import synthetic as S
+    from gbx_lm_amd.batching import BatchScheduler
+    dev = torch.device("cuda", 0)
+    torch.cuda.set_device(dev)
+
+    def clock(fn, reps):
+        fn()
+        torch.cuda.synchronize()
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record()
+        for _ in range(reps):
+            fn()
+        e1.record()
+        torch.cuda.synchronize()
+        return e0.elapsed_time(e1) / reps
+
+    def legs(model, vocab, tag, res):
+        toks = lambda n, o=0: [(o + i * 7919) % vocab for i in range(n)]
+        for T in (512, 4096):
+            def prefill():
+                eng = BatchScheduler(model)
+                eng.step([("p", toks(T))])
+            res[f"{tag}prefill_T{T}_tok_s"] = round(T / clock(prefill, 3) * 1e3)
+        for B, ctx in ((1, 2048), (32, 256)):
+            eng = BatchScheduler(model)
+            eng.step([(i, toks(ctx, i)) for i in range(B)])
+            state = {"t": 0}
+            def decode():
+                state["t"] += 1
+                eng.step([(i, [(state["t"] * 31 + i) % vocab]) for i in range(B)])
+            res[f"{tag}decode_B{B}_ctx{ctx}_tok_s"] = round(B / clock(decode, 64) * 1e3)
+            del eng
+        print(tag or "laruzen", res, file=sys.stderr, flush=True)
+
+    out = {}
+    for name in args.sizes.split(","):
+        g = LARUZEN_SIZES[name]
+        res = {"geometry": g}
+        cfg = S.laruzen_config(**g)
+        model = S.build_laruzen(cfg, device=dev, seed=0)
+        legs(model, cfg["vocab"], "", res)
+        del model
+        torch.cuda.empty_cache()
+        a, m = g["gla"], g["moe"]
+        tm = S.build_tugolix(S.tugolix_config(width=g["width"], delta=dict(heads=2 * a["heads"], kv_heads=a["heads"], dim=a["dim"], vdim=a["dim"], conv=4),
+                                              gla=a, latent=dict(heads=g["left"]["heads"], dim=g["left"]["dim"], vdim=g["left"]["vdim"], kv_rank=512),
+                                              ff=g["ff"], moe=dict(experts=m["experts"], top=m["top"], ff=m["ff"], groups=(8, 4)), pattern="gdlg",
+                                              streams=None, vocab=cfg["vocab"]), device=dev, seed=0)
+        legs(tm, cfg["vocab"], "tugolix_", res)
+        del tm
+        torch.cuda.empty_cache()
+        out[name] = res
+    print(json.dumps({"metric": "laruzen_throughput", "unit": "tokens/s", "dtype": "bf16", "data": "synthetic", "sizes": out}))
+
+
 def main():
     ap = argparse.ArgumentParser()
-    ap.add_argument("--design", default=None, choices=["revitar", "radenex", "tugolix"], help="side benchmark of one model design beside the closest existing "
+    ap.add_argument("--design", default=None, choices=["revitar", "radenex", "tugolix", "laruzen"], help="side benchmark of one model design beside the closest existing "
                     "family at equal size (own JSON line; the default workload and its output are unchanged)")
     ap.add_argument("--sizes", default=None, help="--design: comma-separated names of REVITAR_SIZES (default small,a3b-like) / RADENEX_SIZES "
                     "(default small,lite-like) / TUGOLIX_SIZES (default small,a3b-like)")
@@ -723,8 +799,8 @@ def main():
     if args.design is not None:
         if not torch.cuda.is_available():
             raise SystemExit("bench.py needs an MI355X")
-        args.sizes = args.sizes or {"revitar": "small,a3b-like", "radenex": "small,lite-like", "tugolix": "small,a3b-like"}[args.design]
-        return {"revitar": revitar_bench, "radenex": radenex_bench, "tugolix": tugolix_bench}[args.design](args)
+        args.sizes = args.sizes or {"revitar": "small,a3b-like", "radenex": "small,lite-like", "tugolix": "small,a3b-like", "laruzen": "small,a3b-like"}[args.design]
+        return {"revitar": revitar_bench, "radenex": radenex_bench, "tugolix": tugolix_bench, "laruzen": laruzen_bench}[args.design](args)
     if args.gpus > 1 and "WORLD_SIZE" not in os.environ:
         spawn_ranks(args.gpus)                                     # never returns; nothing has touched the GPU yet
     world = int(os.environ.get("WORLD_SIZE", "1"))

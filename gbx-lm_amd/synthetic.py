@@ -8,6 +8,7 @@ Used by bench.py, the tests and ``__graft_entry__.smoke()``; the layout written 
 from __future__ import annotations
 
 import json
+import math
 import os
 from typing import Dict, Optional
 
@@ -459,6 +460,117 @@ def build_tugolix(config: Dict, device="cpu", seed: int = 0, act_dtype=torch.bfl
     weights = {k: (v.to(act_dtype) if v.is_floating_point() and v.dtype != torch.float32 else v) for k, v in weights.items()}
     with torch.device("meta"):
         model = tugolix.Model(args)
+    model = model.to_empty(device=device)
+    skipped = load_weights(model, weights, device=device)
+    if skipped:
+        raise ValueError(f"tensors without a place in the model: {skipped[:3]}")
+    model.eval()
+    return model
+
+
+# ------------------------------------------------------------------------------------------------ Laruzen (sandwich norms, token shift, linear-attention and parallel mixers)
+def laruzen_config(width: int, gla: Dict, lightning: Dict, left: Dict, right: Dict, ff: int, moe: Dict, pattern: str = "glpg", vocab: int = 32000,
+                   pair: Optional[Dict] = None) -> Dict:
+    """config.json of a Laruzen model: ``pattern`` names the layers in order ('g' gated linear attention, 'l' lightning attention, 'p' the
+    parallel pair of windowed sink attention and a gated linear recurrent unit); the first layer has the dense feed-forward of ``ff``
+    channels, the others the routed one.  ``gla``: heads, dim, vdim, tau; ``lightning``: heads, dim, vdim (decays spread over the
+    heads); ``left``: heads, kv_heads, dim, vdim, window, rot_dims; ``right``: width, blocks, conv; ``moe``: experts, top, ff, shared."""
+    routed = {"kind": "moe", "expert": {"ff": moe["ff"]}, "router": {"experts": moe["experts"], "top": moe["top"]},
+              "shared": {"ff": moe["shared"]} if moe.get("shared") else None}
+    layers = []
+    for i, c in enumerate(pattern):
+        if c == "g":
+            layer = {"type": "gla", "mixer": {k: gla[k] for k in ("heads", "dim", "vdim", "tau")}}
+        elif c == "l":
+            h = lightning["heads"]
+            layer = {"type": "lightning", "mixer": dict({k: lightning[k] for k in ("heads", "dim", "vdim")},
+                                                        decay=[math.exp(-2.0 ** (-1 - 6.0 * j / max(h - 1, 1))) for j in range(h)])}
+        elif c == "p":
+            l = {"heads": left["heads"], "kv_heads": left["kv_heads"], "dim": left["dim"], "vdim": left["vdim"], "scale": left["dim"] ** -0.5,
+                 "mask": {"size": left["window"]},
+                 "rot": {"dims": left.get("rot_dims", left["dim"]), "base": 1e6, "scaling": {"factor": 4.0, "original": 4096, "fast": 32.0, "slow": 1.0}}}
+            layer = {"type": "parallel", "mixer": {"left": l, "right": {k: right[k] for k in ("width", "blocks", "conv")}}}
+        else:
+            raise ValueError(f"laruzen_config: unknown layer letter {c!r}")
+        layer["mlp"] = {"kind": "dense", "ff": ff} if i == 0 else json.loads(json.dumps(routed))
+        layers.append(layer)
+    pair = pair if pair is not None else {"buckets": 65521, "mul_prev": 1000003, "mul_cur": 31}
+    return {"architecture": "Laruzen", "vocab": vocab, "width": width, "norm": {"eps": 1e-6}, "embedding": {"bigram": pair}, "layers": layers}
+
+
+def laruzen_checkpoint(config: Dict, device="cpu", seed: int = 0, decay_rank: int = 16, dtype=torch.bfloat16) -> Dict[str, torch.Tensor]:
+    """Random tensors in the design's checkpoint names with real shapes, generated directly on ``device``."""
+    device = torch.device(device)
+    gen = torch.Generator(device=device)
+    gen.manual_seed(seed)
+    W = config["width"]
+
+    def mat(o, i, mult=1.0):
+        return (torch.randn((o, i), device=device, generator=gen) * (mult * i ** -0.5)).to(dtype)
+
+    def vec(n, lo, hi):
+        return (torch.rand((n,), device=device, generator=gen) * (hi - lo) + lo).to(dtype)
+
+    w = {"embed": torch.randn((config["vocab"], W), device=device, generator=gen).to(dtype), "final.norm": vec(W, -0.1, 0.1), "head": mat(config["vocab"], W)}
+    pair = (config.get("embedding") or {}).get("bigram")
+    if pair:
+        w["bigram"] = torch.randn((pair["buckets"] + 1, W), device=device, generator=gen).to(dtype)
+    for i, layer in enumerate(config["layers"]):
+        p, m, kind = f"l{i}.", layer["mixer"], layer["type"]
+        for nm in ("norm1", "norm1b") + (("norm2", "norm2b") if layer.get("mlp") is not None else ()):
+            w[p + nm] = vec(W, -0.1, 0.1)
+        w[p + "shift"] = vec(W, 0.0, 1.0)
+        x = p + "mix."
+        if kind in ("gla", "lightning"):
+            H, d, dv = m["heads"], m["dim"], m["vdim"]
+            w[x + "q"], w[x + "k"], w[x + "v"], w[x + "g"], w[x + "o"] = mat(H * d, W), mat(H * d, W), mat(H * dv, W), mat(H * dv, W), mat(W, H * dv)
+            if kind == "gla":
+                w[x + "a1"], w[x + "a2"], w[x + "a2.b"], w[x + "norm"] = mat(decay_rank, W), mat(H * d, decay_rank), vec(H * d, 0.0, 5.0), vec(dv, 0.9, 1.1)
+            else:
+                w[x + "norm"] = vec(H * dv, 0.9, 1.1)
+        else:
+            l, r = m["left"], m["right"]
+            H, G, d, dv = l["heads"], l.get("kv_heads", l["heads"]), l["dim"], l["vdim"]
+            a, b = x + "left.", x + "right."
+            w[a + "q"], w[a + "k"], w[a + "v"], w[a + "g"], w[a + "o"] = mat(H * d, W), mat(G * d, W), mat(G * dv, W), mat(H * dv, W), mat(W, H * dv)
+            w[a + "q.b"], w[a + "k.b"], w[a + "v.b"], w[a + "o.b"] = vec(H * d, -0.1, 0.1), vec(G * d, -0.1, 0.1), vec(G * dv, -0.1, 0.1), vec(W, -0.1, 0.1)
+            w[a + "q.norm"], w[a + "k.norm"], w[a + "sink"] = vec(d, 0.9, 1.1), vec(d, 0.9, 1.1), vec(H, -1.0, 1.0)
+            C, nb, taps = r["width"], r["blocks"], r["conv"]
+            bs = C // nb
+            w[b + "x"], w[b + "y"], w[b + "o"], w[b + "x.b"], w[b + "y.b"] = mat(C, W), mat(C, W), mat(W, C), vec(C, -0.1, 0.1), vec(C, -0.1, 0.1)
+            w[b + "conv"], w[b + "conv.b"] = (torch.randn((C, taps), device=device, generator=gen) * 0.5 + 0.25).to(dtype), vec(C, -0.1, 0.1)
+            for nm in ("ra", "ri"):
+                w[b + nm] = (torch.randn((nb, bs, bs), device=device, generator=gen) * bs ** -0.5).to(dtype)
+                w[b + nm + ".b"] = (torch.rand((nb, bs), device=device, generator=gen) - 0.5).to(dtype)
+            w[b + "lam"] = vec(C, -5.0, 0.0)
+            w[x + "left.out"], w[x + "right.out"] = vec(W, 0.9, 1.1), vec(W, 0.9, 1.1)
+        ff, f = layer.get("mlp"), p + "mlp."
+        if ff is not None and ff["kind"] == "dense":
+            n = ff["ff"]
+            w[f + "gate"], w[f + "up"], w[f + "down"] = mat(n, W), mat(n, W), mat(W, n)
+        elif ff is not None:
+            n, E = ff["expert"]["ff"], ff["router"]["experts"]
+            w[f + "router"] = mat(E, W, 2.0)
+            for e in range(E):
+                w[f + f"e{e}.gate"], w[f + f"e{e}.up"], w[f + f"e{e}.down"] = mat(n, W), mat(n, W), mat(W, n)
+            if ff.get("shared"):
+                s = ff["shared"]["ff"]
+                w[f + "shared.gate"], w[f + "shared.up"], w[f + "shared.down"] = mat(s, W), mat(s, W), mat(W, s)
+    return w
+
+
+def build_laruzen(config: Dict, device="cpu", seed: int = 0, act_dtype=torch.bfloat16, decay_rank: int = 16):
+    """Random-init Laruzen with real shapes: a random checkpoint generated on ``device`` goes through the model's own ``sanitize``."""
+    from .models import laruzen
+    from .utils import load_weights
+    device = torch.device(device)
+    weights = laruzen_checkpoint(config, device, seed, decay_rank)
+    args = laruzen.ModelArgs.from_dict(dict(config, shapes=laruzen.Model.shapes_from(weights, config)))
+    model = laruzen.Model(args)                   # (the buffers the constructors compute -- rates, frequency tables -- are tiny)
+    weights = model.sanitize(weights)
+    weights = {k: (v.to(act_dtype) if v.is_floating_point() and v.dtype != torch.float32 else v) for k, v in weights.items()}
+    with torch.device("meta"):
+        model = laruzen.Model(args)
     model = model.to_empty(device=device)
     skipped = load_weights(model, weights, device=device)
     if skipped:
