@@ -3,14 +3,14 @@
 //
 //   causal_conv_rows_kernel    short causal convolution over time per channel with a bias, fp32 out; inputs before the step come from
 //                              the slot's tail, zeros before the sequence.
-//   block_gate_logits_kernel   the two gates' block-diagonal products for steps of few rows: a workgroup per (row, block), the block's
-//                              inputs in LDS, a wave per output row of the matrix (lanes across the inputs, 16-byte loads), fp32 sums
-//                              in a fixed order.  (Prompt-sized steps take a batched fp32 matrix product of the vendor library.)
+//   block_gate_logits_kernel   the two gates' block-diagonal products for steps of few rows: workgroups per (row, block, share of the
+//                              output rows), the block's inputs in LDS, a wave per output row of the matrix (lanes across the inputs,
+//                              16-byte loads), fp32 sums in a fixed order.  (Prompt-sized steps take a batched fp32 matrix product of the vendor library.)
 //   gated_lru_scan_kernel      a = exp(-rate sigmoid(r) softplus(lam)), S <- a S + sqrt(1 - a^2) sigmoid(i) u, out = S gelu(y).  A workgroup
 //                              owns CB channels of one sequence and walks its rows in chunks of CH tokens: all threads form (a, input)
 //                              of the chunk in parallel into LDS, CB threads run the recurrence over the chunk (two LDS reads and one
-//                              multiply-add per token), all threads form the gelu branch and the product.  The next chunk's operands
-//                              are loaded while the recurrence runs.
+//                              multiply-add per token, operands read eight tokens ahead), all threads form the product with the gelu
+//                              branch.  All of the next chunk's operands are loaded while the recurrence runs.
 #include "mixers_common.h"
 
 namespace gbxm {
@@ -40,7 +40,8 @@ __global__ __launch_bounds__(NT) void causal_conv_rows_kernel(const T* __restric
   }
 }
 
-// grid (rows, blocks).  LDS: the block's bs inputs.
+// grid (rows, blocks, splits of the block's output rows).  LDS: the block's bs inputs.  A wave owns one output row at a time, lanes
+// across its inputs with 16-byte loads where the block size allows; the splits spread a step of few rows over the chip.
 template <typename T>
 __global__ __launch_bounds__(NT) void block_gate_logits_kernel(const float* __restrict__ u, const T* __restrict__ w, const float* __restrict__ bias,
                                                               float* __restrict__ logits, int blocks, int bs, int n_out) {
@@ -53,17 +54,28 @@ __global__ __launch_bounds__(NT) void block_gate_logits_kernel(const float* __re
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   const T* wb = w + static_cast<int64_t>(b) * n_out * bs;
   float* lr = logits + (t * blocks + b) * n_out;
-  for (int o = wave; o < n_out; o += NW) {
+  constexpr int PER = 16 / sizeof(T);
+  const bool vec = bs % PER == 0;                  // rows then start 16-byte aligned
+  for (int o = blockIdx.z * NW + wave; o < n_out; o += gridDim.z * NW) {
     const T* wr = wb + static_cast<int64_t>(o) * bs;
     float s = 0.f;
-    for (int i = lane; i < bs; i += 64) s += to_f32(wr[i]) * ub[i];
+    if (vec) {
+      for (int i = lane * PER; i < bs; i += 64 * PER) {
+        T v[PER];
+        *reinterpret_cast<uint4*>(v) = *reinterpret_cast<const uint4*>(wr + i);
+#pragma unroll
+        for (int j = 0; j < PER; ++j) s += to_f32(v[j]) * ub[i + j];
+      }
+    } else {
+      for (int i = lane; i < bs; i += 64) s += to_f32(wr[i]) * ub[i];
+    }
     s = wave_sum(s);
     if (lane == 0) lr[o] = s + bias[b * n_out + o];
   }
 }
 
-constexpr int CB = 32;             // channels of a workgroup
-constexpr int CH = 32;             // tokens of a chunk
+constexpr int CB = 16;             // channels of a workgroup
+constexpr int CH = 64;             // tokens of a chunk
 constexpr int PER = CB * CH / NT;  // elements of a chunk per thread
 
 template <bool FAST> __device__ __forceinline__ float gelu_tanh_(float z) {
@@ -91,6 +103,7 @@ __global__ __launch_bounds__(NT) void gated_lru_scan_kernel(const float* __restr
   float S = 0.f;
   if (threadIdx.x < CB) { S = st[cc]; S = pos0 > 0 ? S : 0.f; }
   float lr[PER], li[PER], uu[PER];
+  T yy[PER];
   auto fetch = [&](int t0) {
 #pragma unroll
     for (int k = 0; k < PER; ++k) {
@@ -100,6 +113,7 @@ __global__ __launch_bounds__(NT) void gated_lru_scan_kernel(const float* __restr
       lr[k] = lp[ci];
       li[k] = lp[bs + ci];
       uu[k] = u[row * C + cc];
+      yy[k] = y[row * y_stride + cc];
     }
   };
   fetch(0);
@@ -112,13 +126,25 @@ __global__ __launch_bounds__(NT) void gated_lru_scan_kernel(const float* __restr
       a_l[tt][cl] = a;
       in_l[tt][cl] = sqrtf(fmaxf(1.f - a * a, 0.f)) * (ig * uu[k]);
     }
+    float g[PER];                                   // the other branch of this chunk, before its operands are replaced by the next chunk's
+#pragma unroll
+    for (int k = 0; k < PER; ++k) g[k] = gelu_tanh_<FAST>(to_f32(yy[k]));
     __syncthreads();
     if (t0 + CH < n) fetch(t0 + CH);
     const int cn = min(CH, n - t0);
     if (threadIdx.x < CB) {
-      for (int tt = 0; tt < cn; ++tt) {
-        S = a_l[tt][cl] * S + in_l[tt][cl];
-        in_l[tt][cl] = S;
+      // eight tokens' operands are read before the eight dependent multiply-adds (LDS latency once per eight, not per token)
+      for (int t8 = 0; t8 < cn; t8 += 8) {
+        float a8[8], i8[8];
+#pragma unroll
+        for (int j = 0; j < 8; ++j) { a8[j] = a_l[t8 + j][cl]; i8[j] = in_l[t8 + j][cl]; }
+#pragma unroll
+        for (int j = 0; j < 8; ++j) {
+          if (t8 + j < cn) S = a8[j] * S + i8[j];
+          i8[j] = S;
+        }
+#pragma unroll
+        for (int j = 0; j < 8; ++j) in_l[t8 + j][cl] = i8[j];
       }
     }
     __syncthreads();
@@ -127,7 +153,7 @@ __global__ __launch_bounds__(NT) void gated_lru_scan_kernel(const float* __restr
       const int tt = tl0 + k * (NT / CB);
       if (tt < cn && live) {
         const int64_t row = row0 + t0 + tt;
-        out[row * C + c] = from_f32<T>(in_l[tt][cl] * gelu_tanh_<FAST>(to_f32(y[row * y_stride + c])));
+        out[row * C + c] = from_f32<T>(in_l[tt][cl] * g[k]);
       }
     }
     __syncthreads();
@@ -172,8 +198,12 @@ int gbxm_block_gate_logits(const float* u, const void* w, const float* bias, flo
   if (bs > 12288) return fail(GBXM_ERR_UNSUPPORTED, "block_gate_logits: blocks of %d channels (at most 12288)", bs);
   if (T_ == 0) return GBXM_OK;
   hipStream_t s = static_cast<hipStream_t>(stream);
-  GBXM_DISPATCH(act, (block_gate_logits_kernel<T><<<dim3(T_, blocks), NT, bs * sizeof(float), s>>>(u, static_cast<const T*>(w), bias, logits, blocks, bs,
-                                                                                                    n_out)));
+  int64_t splits = (512 + T_ * blocks - 1) / (T_ * blocks);      // enough workgroups for the chip, a wave keeps at least one output row
+  const int64_t most = (n_out + NW - 1) / NW;
+  if (splits > most) splits = most;
+  if (splits < 1) splits = 1;
+  GBXM_DISPATCH(act, (block_gate_logits_kernel<T><<<dim3(T_, blocks, static_cast<unsigned>(splits)), NT, bs * sizeof(float), s>>>(
+                         u, static_cast<const T*>(w), bias, logits, blocks, bs, n_out)));
   return after_launch("block_gate_logits");
 }
 
