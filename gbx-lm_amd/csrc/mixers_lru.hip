@@ -161,6 +161,32 @@ __global__ __launch_bounds__(NT) void gated_lru_scan_kernel(const float* __restr
   if (threadIdx.x < CB && live) st[c] = S;
 }
 
+// Steps in which every sequence brings one row: a thread per (sequence, channel), the same arithmetic in the same order.
+template <typename T, bool FAST>
+__global__ __launch_bounds__(NT) void gated_lru_step_kernel(const float* __restrict__ u, const float* __restrict__ logits, int64_t lg_t, int64_t lg_b,
+                                                           const float* __restrict__ lam_sp, const T* __restrict__ y, int64_t y_stride,
+                                                           float* __restrict__ state, T* __restrict__ out, const int* __restrict__ seq, int C, int bs,
+                                                           float rate) {
+  const int b = blockIdx.y;
+  const int c = blockIdx.x * NT + threadIdx.x;
+  if (c >= C) return;
+  const int slot = seq[4 * b], pos0 = seq[4 * b + 1];
+  const int64_t row = seq[4 * b + 3];
+  const int blk = c / bs, ci = c - blk * bs;
+  const float* lp = logits + row * lg_t + static_cast<int64_t>(blk) * lg_b;
+  const float lr = lp[ci], li = lp[bs + ci], uu = u[row * C + c], sp = lam_sp[c];
+  const float yv = to_f32(y[row * y_stride + c]);
+  float* st = state + static_cast<int64_t>(slot) * C + c;
+  float S = *st;
+  S = pos0 > 0 ? S : 0.f;
+  const float r = sigmoid_<FAST>(lr), ig = sigmoid_<FAST>(li);
+  const float a = exp_<FAST>(-rate * r * sp);
+  const float in = sqrtf(fmaxf(1.f - a * a, 0.f)) * (ig * uu);
+  S = a * S + in;
+  *st = S;
+  out[row * C + c] = from_f32<T>(S * gelu_tanh_<FAST>(yv));
+}
+
 bool act_ok(int act) { return act == GBXM_BF16 || act == GBXM_F32; }
 
 }  // namespace
@@ -215,6 +241,16 @@ int gbxm_gated_lru_scan(const float* u, const float* logits, int64_t lg_t, int64
   if (B == 0 || T_ == 0) return GBXM_OK;
   if (B > 65535) return fail(GBXM_ERR_UNSUPPORTED, "gated_lru_scan: more than 65535 sequences in a step");
   hipStream_t s = static_cast<hipStream_t>(stream);
+  if (T_ == B) {                                   // every sequence brings one row
+    const dim3 sgrid((C + NT - 1) / NT, B);
+    if (act == GBXM_BF16)
+      gated_lru_step_kernel<bf16_t, false><<<sgrid, NT, 0, s>>>(u, logits, lg_t, lg_b, lam_sp, static_cast<const bf16_t*>(y), y_stride, state,
+                                                              static_cast<bf16_t*>(out), seq, C, bs, rate);
+    else
+      gated_lru_step_kernel<float, false><<<sgrid, NT, 0, s>>>(u, logits, lg_t, lg_b, lam_sp, static_cast<const float*>(y), y_stride, state,
+                                                             static_cast<float*>(out), seq, C, bs, rate);
+    return after_launch("gated_lru_scan");
+  }
   const dim3 grid((C + CB - 1) / CB, B);
   if (act == GBXM_BF16)
     gated_lru_scan_kernel<bf16_t, false><<<grid, NT, 0, s>>>(u, logits, lg_t, lg_b, lam_sp, static_cast<const bf16_t*>(y), y_stride, state,
