@@ -303,7 +303,7 @@ def radenex_config(width: int, latent: Dict, attention: Dict, ff: int, pattern: 
            "mixer": {"heads": latent["heads"], "dim": latent["dim"], "rot_dim": latent["rot_dim"], "vdim": latent["vdim"],
                      "kv_rank": latent["kv_rank"], "scale": (latent["dim"] + latent["rot_dim"]) ** -0.5,
                      "rot": {"base": 10000.0, "dims": latent["rot_dim"],
-                             "scaling": {"factor": 4.0, "original": 4096, "fast": 32.0, "slow": 1.0}}},
+                             "scaling": {"factor": 8.0, "original": 4096, "fast": 32.0, "slow": 1.0}}},
            "mlp": {"kind": "dense", "ff": ff}}
     att = {"type": "attention",
            "mixer": {"heads": attention["heads"], "kv_heads": attention["kv_heads"], "dim": attention["dim"], "vdim": attention["vdim"],
@@ -488,7 +488,7 @@ def laruzen_config(width: int, gla: Dict, lightning: Dict, left: Dict, right: Di
         elif c == "p":
             l = {"heads": left["heads"], "kv_heads": left["kv_heads"], "dim": left["dim"], "vdim": left["vdim"], "scale": left["dim"] ** -0.5,
                  "mask": {"size": left["window"]},
-                 "rot": {"dims": left.get("rot_dims", left["dim"]), "base": 1e6, "scaling": {"factor": 4.0, "original": 4096, "fast": 32.0, "slow": 1.0}}}
+                 "rot": {"dims": left.get("rot_dims", left["dim"]), "base": 1e6, "scaling": {"factor": 8.0, "original": 4096, "fast": 32.0, "slow": 1.0}}}
             layer = {"type": "parallel", "mixer": {"left": l, "right": {k: right[k] for k in ("width", "blocks", "conv")}}}
         else:
             raise ValueError(f"laruzen_config: unknown layer letter {c!r}")

@@ -5,7 +5,6 @@ between layers of one model and include the corners: grouped and ungrouped key h
 YaRN, windows shorter and longer than the sequences, convolutions of 1 to 4 taps, one gate block and several, head sizes off every
 grid, top 1, no shared expert, layers without a feed-forward, a model without the pair embedding, a parallel layer first."""
 import json
-import math
 import os
 import subprocess
 import sys
@@ -15,13 +14,10 @@ import torch
 
 import laruzen_oracle as O
 from gbx_lm_amd.batching import BatchScheduler, StepBatch
-from gbx_lm_amd.models import gated_lru as LRU
-from gbx_lm_amd.models import recurrent_mixers as RM
-from gbx_lm_amd.models.cache import CacheGroup, SequenceSlots, SlotRowCache
+from gbx_lm_amd.models.cache import SequenceSlots, SlotRowCache
 from gbx_lm_amd.models.embedding import HashedPairEmbedding
-from gbx_lm_amd.models.feed_forward import GatedDenseFeedForward, gate_mul, glu_
+from gbx_lm_amd.models.feed_forward import gate_mul, glu_
 from gbx_lm_amd.models.laruzen import SharedExpertMoE
-from gbx_lm_amd.models.parallel_mixers import ParallelMixers
 from gbx_lm_amd.models.residual import branch_norm_add_norm_, norm_token_shift, normed_pair_mean
 from gbx_lm_amd.models.sink_attention import NORM_UNIT, NORM_WEIGHT, GatedSinkWindowAttention, HeadSegment, rotate_norm_heads_
 from gbx_lm_amd.utils import generate_step, load_model
